@@ -1,4 +1,5 @@
 from .base import ConfigError, KeyReader, read_json
+from .kezolix import KezolixConfig
 from .nebanex import NebanexConfig
 from .pekasun import PekasunConfig
 from .qwen2 import Qwen2Config
@@ -16,6 +17,7 @@ __all__ = [
     "Architecture",
     "ConfigError",
     "KeyReader",
+    "KezolixConfig",
     "NebanexConfig",
     "PekasunConfig",
     "Qwen2Config",

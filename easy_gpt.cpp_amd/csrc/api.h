@@ -154,13 +154,15 @@ int egpt_sigmoid_gate(const void* x, int heads, const void* gate, int gate_split
 // Attention with key size dk and value size dv, a window that keeps the first keep_first tokens visible, and an
 // optional sink per query head (float32 [nq], null: none) in the softmax's denominator, and an optional bias by
 // head and distance (dist_bias float32 [nq][dist_far + 1], null: none): key j of a query at position p gets
-// dist_bias[head][min(p - j, dist_far)] added to its scaled score.  q [n_tokens][nq][dk],
+// dist_bias[head][min(p - j, dist_far)] added to its scaled score.  block > 0: key j is seen only if it lies in the
+// query's block of positions, floor(j / block) == floor(p / block).  slopes float32 [nq] (null: none): the scaled score
+// of key j loses slopes[head] * (p - j) (the matrix-core kernel takes a bias table or slopes, not both).  q [n_tokens][nq][dk],
 // out [n_tokens][nq][dv]; the other operands as egpt_paged_attention.
 int egpt_window_attention(const void* q, void* out, const void* k_cache, const void* v_cache, const int32_t* block_table,
                           int table_width, const int32_t* q_start, const int32_t* q_len, const int32_t* kv_len,
                           int n_seqs, int n_tokens, int nq, int nkv, int dk, int dv, int page_size, float scale,
-                          int window, int keep_first, const float* sink, const float* dist_bias, int dist_far, int dtype,
-                          void* stream);
+                          int window, int keep_first, const float* sink, const float* dist_bias, int dist_far, int block,
+                          const float* slopes, int dtype, void* stream);
 // The same on the matrix cores: dk a multiple of 4 (float32) or 8 (bfloat16) up to 256, dv a multiple of 16 up to 256,
 // page_size a multiple of 16.  row_tiles: tiles of 16 rows to a workgroup of four wavefronts: 8 (32 rows to a wavefront)
 // or 4 (16).  With
@@ -170,7 +172,8 @@ int egpt_window_attention_tiled(const void* q, void* out, float* part_o, float* 
                                 const void* v_cache, const int32_t* block_table, int table_width, const int32_t* q_start,
                                 const int32_t* q_len, const int32_t* kv_len, int n_seqs, int n_tokens, int nq, int nkv,
                                 int dk, int dv, int page_size, float scale, int window, int keep_first, const float* sink,
-                                const float* dist_bias, int dist_far, int n_splits, int row_tiles, int dtype, void* stream);
+                                const float* dist_bias, int dist_far, int block, const float* slopes, int n_splits,
+                                int row_tiles, int dtype, void* stream);
 // ---- residual stream and logits (stream_ops.hip)
 // out[t] = table[ids[t]] * factor as the float32 residual stream.
 int egpt_embed_scaled(const int32_t* ids, const void* table, float factor, float* out, int n_tokens, int hidden, int vocab,
@@ -184,6 +187,15 @@ int egpt_add_layernorm(float* h, const void* delta, int delta_splits, int delta_
 int egpt_normed_pair_mean(const void* a, int a_splits, const void* b, int b_splits, const void* bias_a, const void* bias_b,
                           const void* wa, const void* wb, float eps, float factor, float* out, int n_rows, int hidden,
                           int dtype, void* stream);
+// out[t] = table[ids[t]] + pos_table[positions[t]] as the float32 residual stream.
+int egpt_embed_positions(const int32_t* ids, const int32_t* positions, const void* table, const void* pos_table, float* out,
+                         int n_tokens, int hidden, int vocab, int max_pos, int dtype, void* stream);
+// x = h + mult * LN(y) * post_w (LN without bias; y a product: one tensor or float32 partial sums).  With hist (float32
+// [n_hist + 1][n_rows][hidden]) x is stored as hist[n_hist] and v = sum_(j <= n_hist) mix[j] * hist[j], else v = x.
+// h_out = v (h_out may be h).  With next_w, out = LN(v) * next_w in the activation type.
+int egpt_post_norm_add(const float* h, const void* y, int y_splits, const void* post_w, float eps, float mult, float* hist,
+                       int n_hist, const float* mix, float* h_out, const void* next_w, void* out, int n_rows, int hidden,
+                       int dtype, void* stream);
 // x = cap * tanh(x / cap) in place.
 int egpt_tanh_cap(float* x, float cap, long long n, void* stream);
 // ---- head_prep.hip: norms over a whole projection, a position factor on the queries, the store into pages
@@ -192,27 +204,34 @@ int egpt_whole_norm_store(const void* proj, int n_splits, int row_width, const v
                           int every, const int32_t* slots, void* k_cache, void* v_cache, int n_tokens, int nq, int nkv,
                           int dk, int dv, int page_size, int dtype, void* stream);
 // out = per-head rmsnorm(x) * weight[dv] * silu(gate columns gate_off.. of a product row); x float32 [n_tokens][heads][dv]
-// (x_splits 0) or partial sums [x_splits][n_tokens][heads][dv]
+// (x_splits 0) or partial sums [x_splits][n_tokens][heads][dv]; gate null: no gate
 int egpt_head_norm_gate(const float* x, int x_splits, const void* weight, float eps, const void* gate, int gate_splits, int gate_width,
                         int gate_off, void* out, int n_tokens, int heads, int dv, int dtype, void* stream);
 // ---- linear_recurrence.hip: a matrix state per head that decays per key channel
 // decay[t][c] = sigmoid(z)^(1 / tau), z = bias[c] + sum_r w[c][r] * low[t][r]; low: columns low_off.. of a product row.
 int egpt_channel_decay(const void* low, int low_splits, int low_width, int low_off, int rank, const void* w, const void* bias,
                        float tau, float* decay, int n_tokens, int channels, int dtype, void* stream);
+// gate[t][c] = lower[c] + (1 - lower[c]) * sigmoid(z[t][z_off + c] + bias[c]), float32 (bias, lower may be null: 0).
+int egpt_bounded_gate(const void* z, int z_splits, int z_width, int z_off, const void* bias, const void* lower, float* gate,
+                      int n_tokens, int channels, int dtype, void* stream);
 // S <- diag(decay_t) S + k_t v_t^T, o_t = S^T (q_t * q_scale), token by token for every request of the step; the state
 // float32 [slots][heads][dk][dv] is read from and written to states[slot[b]] (fresh[b] != 0: it starts at zero).
 // q, k, v: columns q_off, k_off, v_off of a product row of proj_width values.  out float32 [egpt_scan_key_splits(dk)][n_tokens][heads][dv]:
-// partial sums over ranges of the key channels, for the consumer to add.
+// partial sums over ranges of the key channels, for the consumer to add.  q_silu: q_t is silu of its columns;
+// tied_keys: k_t = 1 - decay_t (k_off is not read).
 int egpt_scan_key_splits(int dk);
 int egpt_decayed_state_scan(const void* proj, int n_splits, int proj_width, int q_off, int k_off, int v_off, float q_scale,
                             const float* decay, float* states, const int32_t* slots, const unsigned char* fresh,
                             const int32_t* q_start, const int32_t* q_len, int n_seqs, int n_tokens, float* out, int heads,
-                            int dk, int dv, int dtype, void* stream);
+                            int dk, int dv, int q_silu, int tied_keys, int dtype, void* stream);
 // ---- moe.hip: a mixture of gated experts
 // logits = x router^T + bias in float32; the `top` largest per token (lowest index among equals) to chosen[t][top], the
 // softmax over the chosen logits to weight[t][top].
+// score_all: scores = softmax over all experts; the `top` experts with the largest score + correction (float32 [experts],
+// null: none) are chosen, and weigh score / (sum of the chosen scores + 1e-20) * weight_scale.
 int egpt_moe_route(const void* x, const void* router, const void* bias, int32_t* chosen, float* weight, int n_tokens,
-                   int hidden, int experts, int top, int dtype, void* stream);
+                   int hidden, int experts, int top, int score_all, const float* correction, float weight_scale, int dtype,
+                   void* stream);
 // Rows (token, choice) grouped by expert: row_token[n_tokens * top] the token of every grouped row, place[t][top] the
 // grouped row of every (token, choice), tiles[0] the number of row tiles, then per tile (expert, first row, rows).
 // tile_rows: rows to a tile.  tiles holds 1 + 3 * (n_tokens * top / tile_rows + experts + 1) int32.
@@ -222,12 +241,21 @@ int egpt_moe_group(const int32_t* chosen, int32_t* row_token, int32_t* place, in
 // (an expert's gate rows, then its up rows).  act [n_tokens * top][ff] of the activation type.
 int egpt_moe_gate_up(const void* x, const void* w_gate_up, const int32_t* row_token, const int32_t* tiles, void* act,
                      int n_rows, int hidden, int ff, int experts, int tile_rows, int dtype, void* stream);
+// act[row] = relu(x[row_token[row]] Wu_e^T)^2 for every grouped row; w_up [experts][ff][hidden].
+int egpt_moe_up(const void* x, const void* w_up, const int32_t* row_token, const int32_t* tiles, void* act, int n_rows,
+                int hidden, int ff, int experts, int tile_rows, int dtype, void* stream);
 // y[row] = act[row] Wd_e^T, float32 [n_tokens * top][hidden]; w_down [experts][hidden][ff].
 int egpt_moe_down(const void* act, const void* w_down, const int32_t* tiles, float* y, int n_rows, int hidden, int ff,
                   int experts, int tile_rows, int dtype, void* stream);
 // out[t] = sum_c weight[t][c] * y[place[t][c]] in the order of the choices, float32 [n_tokens][hidden].
 int egpt_moe_combine(const float* y, const int32_t* place, const float* weight, float* out, int n_tokens, int top, int hidden,
                      void* stream);
+// ---- activations.hip: what stands between the two products of a feed-forward without a gate
+// out[t][j] = f(z[t][j]) for the first `cols` columns of a product row of z_width values (one tensor or float32 partial sums):
+// mode 0: relu(z)^2; mode 1: the normed polynomial c0 N(z) + c1 N(z^2) + c2 N(z^3) + c3 with N(u) = u / sqrt(mean_j(u_j^2) + eps)
+// over the row's cols values (coef float32 [4]).  gate_col >= 0: times sigmoid(z[t][gate_col]), one number per row.
+int egpt_ff_activation(const void* z, int z_splits, int z_width, int cols, int mode, const float* coef, float eps, int gate_col,
+                       void* out, int n_tokens, int dtype, void* stream);
 // scratch: n_rows * 32 floats followed by n_rows * 32 int32 (two-stage search for wide vocabularies), or null.
 int egpt_argmax(const float* logits, int32_t* out, void* scratch, int n_rows, int vocab, void* stream);
 // egpt_argmax for callers that cannot allocate device memory and have no workspace to pass (code under graph

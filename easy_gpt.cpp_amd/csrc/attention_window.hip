@@ -1,10 +1,13 @@
 // Softmax attention over the paged cache with separate key and value sizes, a window that keeps the first tokens,
-// a sink in the softmax and a learned bias per head and distance; ragged batches (prompt portions and single decoded tokens in one launch).
+// a sink in the softmax, a learned bias per head and distance, keys visible only within the query's own block of
+// positions, and a penalty per head that grows with the distance; ragged batches (prompt portions and single decoded tokens in one launch).
 //
 // Query i of request b stands at position p = kv_len[b] - q_len[b] + i and sees key j if j <= p and
 // (window == 0 or p - j < window or j < keep_first).  score = (q . k) * scale over the key size dk; the softmax is
 // over the visible keys, and with a sink its denominator also holds exp(sink[head]), which has no key and no value
 // and is not scaled; with a distance bias [nq][far + 1] the score of key j gets bias[head][min(p - j, far)] added, unscaled;
+// with block > 0 a key is seen only if floor(j / block) == floor(p / block) (blocks are counted from position 0 of the
+// request, wherever a step cuts it); with slopes [nq] the score of key j loses slopes[head] * (p - j), unscaled;
 // the output is the weighted sum of the values of size dv.  Query head h reads key/value head
 // h / (nq / nkv).  Queries q [T][nq][dk]; keys in pages [page][kv head][offset][dk], values in pages
 // [page][kv head][dv][offset]; nothing that is not visible is read, so pages need no clearing and pages that a window
@@ -23,6 +26,13 @@ __device__ __forceinline__ int request_of(const int32_t* q_start, int n_seqs, in
         const int mid = (lo + hi + 1) / 2;
         if (q_start[mid] <= t) lo = mid; else hi = mid - 1;
     }
+    return lo;
+}
+
+// the lowest key position that a query at position p sees, the kept first tokens aside
+__device__ __forceinline__ int lowest_seen(int p, int window, int block) {
+    int lo = window > 0 ? max(0, p - window + 1) : 0;
+    if (block > 0) lo = max(lo, p / block * block);
     return lo;
 }
 
@@ -72,7 +82,7 @@ __global__ __launch_bounds__(64 * kSimpleWaves) void window_attention_simple_ker
     const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ q_start,
     const int32_t* __restrict__ q_len, const int32_t* __restrict__ kv_len, int n_seqs, int nq, int nkv, int dk, int dv,
     int page_size, float scale, int window, int keep_first, const float* __restrict__ sink,
-    const float* __restrict__ dist_bias, int dist_far) {
+    const float* __restrict__ dist_bias, int dist_far, int block, const float* __restrict__ slopes) {
     constexpr int kMaxOwn = kWidest / kWave;
     __shared__ __attribute__((aligned(16))) float q_s[kWidest];
     __shared__ float part_ml[kSimpleWaves][2];
@@ -81,7 +91,7 @@ __global__ __launch_bounds__(64 * kSimpleWaves) void window_attention_simple_ker
     const int b = request_of(q_start, n_seqs, t);
     if (t - q_start[b] >= q_len[b]) return;                  // a row that belongs to no request
     const int p = kv_len[b] - q_len[b] + (t - q_start[b]);
-    const int lo = window > 0 ? max(0, p - window + 1) : 0;
+    const int lo = lowest_seen(p, window, block);
     const int n_first = min(keep_first, lo);                 // kept first tokens that the window does not hold anyway
     const int n_visible = n_first + (p - lo + 1);
     const int kvh = h / (nq / nkv);
@@ -100,6 +110,7 @@ __global__ __launch_bounds__(64 * kSimpleWaves) void window_attention_simple_ker
             const T* kr = k_cache + ((page * nkv + kvh) * page_size + j % page_size) * dk;
             s = dot_row(q_s, kr, dk) * scale;
             if (dist_bias) s += dist_bias[static_cast<size_t>(h) * (dist_far + 1) + min(p - j, dist_far)];
+            if (slopes) s -= slopes[h] * static_cast<float>(p - j);
         }
         const float m_new = fmaxf(m_run, wave_max(s));       // finite: the chunk's first key is visible
         const float pj = vi < n_visible ? expf(s - m_new) : 0.f;
@@ -223,6 +234,8 @@ struct WindowArgs {
     const float* sink;
     const float* dist_bias;  // [nq][dist_far + 1] or null
     int dist_far;
+    const float* slopes;     // [nq] or null
+    int block;               // keys are seen within the query's block of this many positions (0: no blocks)
     int table_width, n_seqs, n_tokens, nq, nkv, dk, dv, page_size, window, keep_first, n_splits;
     int page_shift;          // log2 of the page size if that is a power of two, else -1
     float scale;
@@ -280,9 +293,9 @@ __global__ __launch_bounds__(64 * RT, (DT * RW <= 8 ? 2 : 1)) void window_attent
     const int blk_first = grp * ROWS, blk_last = min(rows, blk_first + ROWS) - 1;
     const int p_max = kv - n + blk_last / group_size;
     const int p_min = kv - n + blk_first / group_size;
-    const int lo_blk = window > 0 ? max(0, p_min - window + 1) : 0;
+    const int lo_blk = lowest_seen(p_min, window, a.block);
     const int t_begin = lo_blk / KT, t_end = p_max / KT + 1;
-    const int keep = window > 0 ? min(a.keep_first, lo_blk) : 0;     // kept first tokens below the window
+    const int keep = (window > 0 || a.block > 0) ? min(a.keep_first, lo_blk) : 0;     // kept first tokens below the window
     const int kept_chunks = min((keep + KT - 1) / KT, t_begin);
     const int n_chunks = kept_chunks + (t_end - t_begin);
     const int per_split = (n_chunks + a.n_splits - 1) / a.n_splits;
@@ -299,7 +312,7 @@ __global__ __launch_bounds__(64 * RT, (DT * RW <= 8 ? 2 : 1)) void window_attent
         tok[w] = qs + i_tok;
         head[w] = kh * group_size + (valid[w] ? r % group_size : 0);
         p_row[w] = valid[w] ? kv - n + i_tok : -1;
-        lo_row[w] = (window > 0 && valid[w]) ? max(0, p_row[w] - window + 1) : 0;
+        lo_row[w] = valid[w] ? lowest_seen(p_row[w], window, a.block) : 0;
     }
 
     // the smallest position and the largest window start among a tile's rows (rows of no token aside)
@@ -522,6 +535,19 @@ __global__ __launch_bounds__(64 * RT, (DT * RW <= 8 ? 2 : 1)) void window_attent
                         acc[w][kt][v] = sc;
                         mx = fmaxf(mx, sc);
                     }
+            } else if (a.slopes != nullptr) {
+                // the penalty of the row's head times the distance
+                const float slope = a.slopes[head[w]];
+#pragma unroll
+                for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        const int key = key0 + kt * 16 + lg * 4 + v;
+                        const bool seen = whole || (key <= p_row[w] && (key >= lo_row[w] || key < a.keep_first));
+                        const float sc = seen ? fmaf(acc[w][kt][v], scale, -slope * static_cast<float>(p_row[w] - key)) : -INFINITY;
+                        acc[w][kt][v] = sc;
+                        mx = fmaxf(mx, sc);
+                    }
             } else if (whole) {
 #pragma unroll
                 for (int kt = 0; kt < NKT; ++kt)
@@ -708,10 +734,11 @@ extern "C" int egpt_window_attention(const void* q, void* out, const void* k_cac
                                      const int32_t* block_table, int table_width, const int32_t* q_start,
                                      const int32_t* q_len, const int32_t* kv_len, int n_seqs, int n_tokens, int nq,
                                      int nkv, int dk, int dv, int page_size, float scale, int window, int keep_first,
-                                     const float* sink, const float* dist_bias, int dist_far, int dtype, void* stream) {
+                                     const float* sink, const float* dist_bias, int dist_far, int block, const float* slopes,
+                                     int dtype, void* stream) {
     if (!q || !out || !k_cache || !v_cache || !block_table || !q_start || !q_len || !kv_len) return EGPT_BAD_ARGUMENT;
     if (n_seqs <= 0 || n_tokens < 0 || nq <= 0 || nkv <= 0 || nq % nkv != 0 || dk <= 0 || dv <= 0 || page_size <= 0 ||
-        table_width <= 0 || window < 0 || keep_first < 0 || (dtype != 0 && dtype != 1) || (dist_bias && dist_far < 0))
+        table_width <= 0 || window < 0 || keep_first < 0 || (dtype != 0 && dtype != 1) || (dist_bias && dist_far < 0) || block < 0)
         return EGPT_BAD_ARGUMENT;
     if (dk > kWidest || dv > kWidest || nq > 65535) return EGPT_UNSUPPORTED_SIZE;
     if (n_tokens == 0) return EGPT_OK;
@@ -721,12 +748,12 @@ extern "C" int egpt_window_attention(const void* q, void* out, const void* k_cac
         window_attention_simple_kernel<float><<<grid, kWave * kSimpleWaves, 0, s>>>(
             static_cast<const float*>(q), static_cast<float*>(out), static_cast<const float*>(k_cache),
             static_cast<const float*>(v_cache), block_table, table_width, q_start, q_len, kv_len, n_seqs, nq, nkv, dk,
-            dv, page_size, scale, window, keep_first, sink, dist_bias, dist_far);
+            dv, page_size, scale, window, keep_first, sink, dist_bias, dist_far, block, slopes);
     else
         window_attention_simple_kernel<bf16_t><<<grid, kWave * kSimpleWaves, 0, s>>>(
             static_cast<const bf16_t*>(q), static_cast<bf16_t*>(out), static_cast<const bf16_t*>(k_cache),
             static_cast<const bf16_t*>(v_cache), block_table, table_width, q_start, q_len, kv_len, n_seqs, nq, nkv, dk,
-            dv, page_size, scale, window, keep_first, sink, dist_bias, dist_far);
+            dv, page_size, scale, window, keep_first, sink, dist_bias, dist_far, block, slopes);
     EGPT_CHECK_LAUNCH();
     return EGPT_OK;
 }
@@ -736,11 +763,12 @@ extern "C" int egpt_window_attention_tiled(const void* q, void* out, float* part
                                            const int32_t* q_start, const int32_t* q_len, const int32_t* kv_len, int n_seqs,
                                            int n_tokens, int nq, int nkv, int dk, int dv, int page_size, float scale,
                                            int window, int keep_first, const float* sink, const float* dist_bias,
-                                           int dist_far, int n_splits, int row_tiles, int dtype, void* stream) {
+                                           int dist_far, int block, const float* slopes, int n_splits, int row_tiles, int dtype,
+                                           void* stream) {
     if (!q || !out || !k_cache || !v_cache || !block_table || !q_start || !q_len || !kv_len) return EGPT_BAD_ARGUMENT;
     if (n_seqs <= 0 || n_tokens < 0 || nq <= 0 || nkv <= 0 || nq % nkv != 0 || dk <= 0 || dv <= 0 || page_size <= 0 ||
         table_width <= 0 || window < 0 || keep_first < 0 || n_splits < 1 || (dtype != 0 && dtype != 1) ||
-        (row_tiles != 4 && row_tiles != 8) || (dist_bias && dist_far < 0))
+        (row_tiles != 4 && row_tiles != 8) || (dist_bias && dist_far < 0) || block < 0 || (dist_bias && slopes))
         return EGPT_BAD_ARGUMENT;
     if (n_splits > 1 && (!part_o || !part_ml)) return EGPT_BAD_ARGUMENT;
     const int e = dtype == 0 ? 4 : 8;
@@ -750,7 +778,7 @@ extern "C" int egpt_window_attention_tiled(const void* q, void* out, float* part
     WindowArgs a;
     a.q = q; a.out = out; a.part_o = part_o; a.part_ml = part_ml; a.k_cache = k_cache; a.v_cache = v_cache;
     a.block_table = block_table; a.q_start = q_start; a.q_len = q_len; a.kv_len = kv_len; a.sink = sink;
-    a.dist_bias = dist_bias; a.dist_far = dist_far;
+    a.dist_bias = dist_bias; a.dist_far = dist_far; a.slopes = slopes; a.block = block;
     a.table_width = table_width; a.n_seqs = n_seqs; a.n_tokens = n_tokens; a.nq = nq; a.nkv = nkv; a.dk = dk; a.dv = dv;
     a.page_size = page_size; a.window = window; a.keep_first = keep_first; a.n_splits = n_splits; a.scale = scale;
     a.page_shift = -1;

@@ -18,7 +18,7 @@ import time
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 SOURCES = ["elementwise.hip", "gemm.hip", "gemm_skinny.hip", "gemm_gate_up.hip", "attention.hip", "attention_mfma.hip", "attention_any.hip",
-           "attention_window.hip", "head_prep.hip", "sampling.hip", "stream_ops.hip", "linear_recurrence.hip", "moe.hip"]
+           "attention_window.hip", "head_prep.hip", "sampling.hip", "stream_ops.hip", "linear_recurrence.hip", "moe.hip", "activations.hip"]
 HEADERS = ["api.h", "common.h"]
 LIB_NAME = "libeasygpt_hip.so"
 ARCH = "gfx950"

@@ -272,7 +272,7 @@ __global__ __launch_bounds__(256) void whole_norm_store_kernel(
 
 // out[t][h * dv + d] = x[t][h * dv + d] / rms(x[t][h * dv ..]) * weight[d] * silu(g[t][gate_off + h * dv + d]): the
 // RMS norm of every head's float32 output (one tensor, or partial sums that are added here) with a weight that the heads share, and a SiLU gate from columns of a
-// product row.  One wavefront per (token, head).
+// product row (no gate: the normed heads as they are).  One wavefront per (token, head).
 template <typename T>
 __global__ __launch_bounds__(kWave) void head_norm_gate_kernel(ProductView<float> x, const T* __restrict__ weight,
                                                                float eps, ProductView<T> g, int gate_width, int gate_off,
@@ -286,8 +286,11 @@ __global__ __launch_bounds__(kWave) void head_norm_gate_kernel(ProductView<float
     }
     const float inv = inv_rms(wave_sum(ss), 1.0f / static_cast<float>(dv), eps);
     for (int d = lane; d < dv; d += kWave) {
-        const float gate = g.at(static_cast<size_t>(t) * gate_width + gate_off + h * dv + d);
-        const float y = x.at(xr + d) * inv * to_float(weight[d]) * (gate / (1.0f + expf(-gate)));
+        float y = x.at(xr + d) * inv * to_float(weight[d]);
+        if (g.present()) {
+            const float gate = g.at(static_cast<size_t>(t) * gate_width + gate_off + h * dv + d);
+            y *= gate / (1.0f + expf(-gate));
+        }
         out[(static_cast<size_t>(t) * heads + h) * dv + d] = from_float<T>(y);
     }
 }
@@ -419,8 +422,9 @@ extern "C" int egpt_whole_norm_store(const void* proj, int n_splits, int row_wid
                                      const void* q_weight, const void* k_weight, float eps, const int32_t* positions,
                                      float coef, int every, const int32_t* slots, void* k_cache, void* v_cache,
                                      int n_tokens, int nq, int nkv, int dk, int dv, int page_size, int dtype, void* stream) {
-    if (!proj || !q_out || n_splits < 0 || n_tokens < 0 || nq <= 0 || nkv <= 0 || dk <= 0 || dv <= 0 || page_size <= 0 ||
-        every < 0 || (dtype != 0 && dtype != 1))
+    // nkv == 0: a row holds queries alone (a layer that reads keys and values that another layer stored); nothing is stored
+    if (!proj || !q_out || n_splits < 0 || n_tokens < 0 || nq <= 0 || nkv < 0 || dk <= 0 || dv <= 0 || page_size <= 0 ||
+        every < 0 || (dtype != 0 && dtype != 1) || (nkv == 0 && slots))
         return EGPT_BAD_ARGUMENT;
     if (row_width < (nq + nkv) * dk + nkv * dv) return EGPT_BAD_ARGUMENT;
     if (every > 0 && !positions) return EGPT_BAD_ARGUMENT;
@@ -445,9 +449,10 @@ extern "C" int egpt_whole_norm_store(const void* proj, int n_splits, int row_wid
 extern "C" int egpt_head_norm_gate(const float* x, int x_splits, const void* weight, float eps, const void* gate, int gate_splits,
                                    int gate_width, int gate_off, void* out, int n_tokens, int heads, int dv, int dtype,
                                    void* stream) {
-    if (!x || x_splits < 0 || !weight || !gate || !out || n_tokens < 0 || heads <= 0 || dv <= 0 || gate_splits < 0 || gate_off < 0 ||
-        gate_off + heads * dv > gate_width || (dtype != 0 && dtype != 1))
+    if (!x || x_splits < 0 || !weight || !out || n_tokens < 0 || heads <= 0 || dv <= 0 || gate_splits < 0 || (dtype != 0 && dtype != 1))
         return EGPT_BAD_ARGUMENT;
+    if (gate && (gate_off < 0 || gate_off + heads * dv > gate_width)) return EGPT_BAD_ARGUMENT;
+    if (!gate) gate_splits = 0;
     if (heads > 65535) return EGPT_UNSUPPORTED_SIZE;
     if (n_tokens == 0) return EGPT_OK;
     hipStream_t s = static_cast<hipStream_t>(stream);

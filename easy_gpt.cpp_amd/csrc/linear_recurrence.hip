@@ -5,7 +5,9 @@
 // tokens, so the result does not depend on the cut at all.  Decays, the state and the output sum are float32.
 //
 // egpt_channel_decay makes the decays a = sigmoid(z)^(1/tau) from a low-rank projection (z = W low + b);
-// egpt_decayed_state_scan runs the recurrence.
+// egpt_bounded_gate makes decays with a learned lower bound, a = l + (1 - l) sigmoid(z + b), from columns of a product;
+// egpt_decayed_state_scan runs the recurrence; its queries may pass through SiLU on their way in, and its keys may be
+// tied to the decays, k = 1 - a (a forget gate that also sets what is written), instead of columns of the product.
 #include "api.h"
 #include "common.h"
 
@@ -44,6 +46,21 @@ __global__ __launch_bounds__(256) void channel_decay_kernel(ProductView<T> low, 
     }
 }
 
+// a[t][c] = lower[c] + (1 - lower[c]) * sigmoid(z[t][c] + bias[c]), float32; z are columns z_off.. of a product row.
+template <typename T>
+__global__ __launch_bounds__(256) void bounded_gate_kernel(ProductView<T> z, int z_width, int z_off, const T* __restrict__ bias,
+                                                           const T* __restrict__ lower, float* __restrict__ gate, int channels,
+                                                           size_t total) {
+    const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const size_t t = idx / channels;
+    const int c = static_cast<int>(idx % channels);
+    float v = z.at(t * z_width + z_off + c);
+    if (bias) v += to_float(bias[c]);
+    const float low = lower ? to_float(lower[c]) : 0.f;
+    gate[idx] = low + (1.0f - low) * (1.0f / (1.0f + expf(-v)));
+}
+
 constexpr int kScanTokens = 32;     // tokens staged in LDS at a time
 constexpr int kScanCols = 64;       // value channels per workgroup: a lane is a column of the state
 constexpr int kScanKeys = 16;       // key channels per workgroup
@@ -62,7 +79,7 @@ __global__ __launch_bounds__(64 * kScanWaves) void decayed_state_scan_kernel(
     ProductView<T> proj, int proj_width, int q_off, int k_off, int v_off, float q_scale, const float* __restrict__ decay,
     float* __restrict__ states, const int32_t* __restrict__ slots, const unsigned char* __restrict__ fresh,
     const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len, float* __restrict__ out, int n_tokens, int heads,
-    int dk, int dv, int key_splits) {
+    int dk, int dv, int key_splits, int q_silu, int tied_keys) {
     constexpr int NS = kScanWaves, DKR = kScanKeys / kScanWaves, THREADS = 64 * NS, DKP = kScanKeys;
     constexpr int QKA = kScanTokens * DKP / THREADS;          // values of q (or k, or decays) of a batch per thread
     constexpr int VL = kScanTokens * kScanCols / THREADS;     // values of v, and outputs, of a batch per thread
@@ -101,8 +118,8 @@ __global__ __launch_bounds__(64 * kScanWaves) void decayed_state_scan_kernel(
             if (tt < count && r < dk) {
                 const size_t row = static_cast<size_t>(t0 + base + tt);
                 rq[u] = proj.at(row * proj_width + q_off + h * dk + r);      // (scaled when it is staged: nothing here waits for a load)
-                rk[u] = proj.at(row * proj_width + k_off + h * dk + r);
                 ra[u] = decay[row * channels + h * dk + r];
+                if (!tied_keys) rk[u] = proj.at(row * proj_width + k_off + h * dk + r);
             }
         }
 #pragma unroll
@@ -120,8 +137,10 @@ __global__ __launch_bounds__(64 * kScanWaves) void decayed_state_scan_kernel(
         __syncthreads();                          // the batch before is read, its parts are added
 #pragma unroll
         for (int u = 0; u < QKA; ++u) {
-            q_s[tid + u * THREADS] = rq[u] * q_scale;
-            k_s[tid + u * THREADS] = rk[u];
+            // (a tied key is 1 - a; a place that holds no token or no channel has a = 0 and would get k = 1, which meets a
+            // query of zero and a state row that is never stored)
+            q_s[tid + u * THREADS] = (q_silu ? rq[u] / (1.0f + expf(-rq[u])) : rq[u]) * q_scale;
+            k_s[tid + u * THREADS] = tied_keys ? 1.0f - ra[u] : rk[u];
             a_s[tid + u * THREADS] = ra[u];
         }
 #pragma unroll
@@ -186,16 +205,38 @@ extern "C" int egpt_channel_decay(const void* low, int low_splits, int low_width
     return EGPT_OK;
 }
 
+extern "C" int egpt_bounded_gate(const void* z, int z_splits, int z_width, int z_off, const void* bias, const void* lower,
+                                 float* gate, int n_tokens, int channels, int dtype, void* stream) {
+    if (!z || !gate || z_splits < 0 || z_off < 0 || channels <= 0 || z_off + channels > z_width || n_tokens < 0 ||
+        (dtype != 0 && dtype != 1))
+        return EGPT_BAD_ARGUMENT;
+    if (n_tokens == 0) return EGPT_OK;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const size_t stride = static_cast<size_t>(n_tokens) * z_width, total = static_cast<size_t>(n_tokens) * channels;
+    const unsigned blocks = static_cast<unsigned>((total + 255) / 256);
+    if (dtype == 0)
+        bounded_gate_kernel<float><<<blocks, 256, 0, s>>>(scan_view<float>(z, z_splits, stride), z_width, z_off,
+                                                          static_cast<const float*>(bias), static_cast<const float*>(lower), gate,
+                                                          channels, total);
+    else
+        bounded_gate_kernel<bf16_t><<<blocks, 256, 0, s>>>(scan_view<bf16_t>(z, z_splits, stride), z_width, z_off,
+                                                           static_cast<const bf16_t*>(bias), static_cast<const bf16_t*>(lower), gate,
+                                                           channels, total);
+    EGPT_CHECK_LAUNCH();
+    return EGPT_OK;
+}
+
 template <typename T>
 static int launch_scan(const void* proj, int n_splits, int proj_width, int q_off, int k_off, int v_off, float q_scale,
                        const float* decay, float* states, const int32_t* slots, const unsigned char* fresh,
                        const int32_t* q_start, const int32_t* q_len, int n_seqs, int n_tokens, float* out, int heads, int dk,
-                       int dv, hipStream_t s) {
+                       int dv, int q_silu, int tied_keys, hipStream_t s) {
     const ProductView<T> view = scan_view<T>(proj, n_splits, static_cast<size_t>(n_tokens) * proj_width);
     const int key_splits = (dk + kScanKeys - 1) / kScanKeys;
     dim3 grid(n_seqs, heads, (dv + kScanCols - 1) / kScanCols * key_splits);
     decayed_state_scan_kernel<T><<<grid, 64 * kScanWaves, 0, s>>>(view, proj_width, q_off, k_off, v_off, q_scale, decay, states, slots,
-                                                                  fresh, q_start, q_len, out, n_tokens, heads, dk, dv, key_splits);
+                                                                  fresh, q_start, q_len, out, n_tokens, heads, dk, dv, key_splits,
+                                                                  q_silu, tied_keys);
     return EGPT_OK;
 }
 
@@ -204,11 +245,12 @@ extern "C" int egpt_scan_key_splits(int dk) { return dk > 0 ? (dk + kScanKeys - 
 extern "C" int egpt_decayed_state_scan(const void* proj, int n_splits, int proj_width, int q_off, int k_off, int v_off,
                                        float q_scale, const float* decay, float* states, const int32_t* slots,
                                        const unsigned char* fresh, const int32_t* q_start, const int32_t* q_len, int n_seqs,
-                                       int n_tokens, float* out, int heads, int dk, int dv, int dtype, void* stream) {
+                                       int n_tokens, float* out, int heads, int dk, int dv, int q_silu, int tied_keys,
+                                       int dtype, void* stream) {
     if (!proj || !decay || !states || !slots || !q_start || !q_len || !out || n_splits < 0 || n_seqs <= 0 || n_tokens < 0 ||
-        heads <= 0 || dk <= 0 || dv <= 0 || q_off < 0 || k_off < 0 || v_off < 0 || (dtype != 0 && dtype != 1))
+        heads <= 0 || dk <= 0 || dv <= 0 || q_off < 0 || (!tied_keys && k_off < 0) || v_off < 0 || (dtype != 0 && dtype != 1))
         return EGPT_BAD_ARGUMENT;
-    if (q_off + heads * dk > proj_width || k_off + heads * dk > proj_width || v_off + heads * dv > proj_width)
+    if (q_off + heads * dk > proj_width || (!tied_keys && k_off + heads * dk > proj_width) || v_off + heads * dv > proj_width)
         return EGPT_BAD_ARGUMENT;
     if (heads > 65535 || static_cast<long long>((dv + kScanCols - 1) / kScanCols) * ((dk + kScanKeys - 1) / kScanKeys) > 65535)
         return EGPT_UNSUPPORTED_SIZE;
@@ -216,10 +258,10 @@ extern "C" int egpt_decayed_state_scan(const void* proj, int n_splits, int proj_
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype == 0)
         launch_scan<float>(proj, n_splits, proj_width, q_off, k_off, v_off, q_scale, decay, states, slots, fresh, q_start,
-                           q_len, n_seqs, n_tokens, out, heads, dk, dv, s);
+                           q_len, n_seqs, n_tokens, out, heads, dk, dv, q_silu, tied_keys, s);
     else
         launch_scan<bf16_t>(proj, n_splits, proj_width, q_off, k_off, v_off, q_scale, decay, states, slots, fresh, q_start,
-                            q_len, n_seqs, n_tokens, out, heads, dk, dv, s);
+                            q_len, n_seqs, n_tokens, out, heads, dk, dv, q_silu, tied_keys, s);
     EGPT_CHECK_LAUNCH();
     return EGPT_OK;
 }

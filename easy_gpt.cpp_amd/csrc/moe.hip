@@ -1,7 +1,9 @@
 // A mixture of gated experts: float32 router with top-k choice, rows grouped by expert on the device, the experts'
 // products as grouped products on the matrix cores, and the weighted sum of a token's choices in a fixed order.
 //
-//   egpt_moe_route     logits = x R^T + b (float32), the `top` largest, softmax over those
+//   egpt_moe_route     logits = x R^T + b (float32), the `top` largest, softmax over those; or the softmax over all
+//                      experts, the choice by score + a correction per expert, the chosen scores over their sum
+//   egpt_moe_up        act = relu(x Wu^T)^2 per grouped row: experts without a gate
 //   egpt_moe_group     (token, choice) rows grouped by expert; tiles of rows, each of one expert
 //   egpt_moe_gate_up   act = silu(x Wg^T) * (x Wu^T) per grouped row, with that row's expert
 //   egpt_moe_down      y = act Wd^T per grouped row (float32)
@@ -57,7 +59,8 @@ template <typename T>
 __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ x, const T* __restrict__ router,
                                                         const T* __restrict__ bias, int32_t* __restrict__ chosen,
                                                         float* __restrict__ weight, int n_tokens, int hidden, int experts,
-                                                        int top) {
+                                                        int top, int score_all, const float* __restrict__ correction,
+                                                        float weight_scale) {
     extern __shared__ float logits_s[];          // [experts]
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
     const int t = blockIdx.x;
@@ -81,6 +84,55 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ x,
     }
     __syncthreads();
     if (wave != 0) return;
+    if (score_all) {
+        // scores s = softmax(z) over all experts; an expert is chosen by s + correction and weighs s over the sum of
+        // the chosen scores.  z[] keeps the choice scores, score_s[] (behind it) the scores themselves.
+        float* score_s = logits_s + experts;
+        float mx = -INFINITY;
+        for (int e = lane; e < experts; e += kWave) mx = fmaxf(mx, z[e]);
+        mx = wave_max(mx);
+        float sum = 0.f;
+        for (int e = lane; e < experts; e += kWave) sum += expf(z[e] - mx);
+        const float inv_sum = 1.0f / wave_sum(sum);
+        for (int e = lane; e < experts; e += kWave) {
+            const float sc = expf(z[e] - mx) * inv_sum;
+            score_s[e] = sc;
+            z[e] = sc + (correction ? correction[e] : 0.f);
+        }
+        float chosen_sum = 0.f;
+        for (int c = 0; c < top; ++c) {
+            float best = -INFINITY;
+            int best_e = 0x7fffffff;
+            for (int e = lane; e < experts; e += kWave) {
+                const float v = z[e];
+                if (v > best || (v == best && e < best_e)) {
+                    best = v;
+                    best_e = e;
+                }
+            }
+#pragma unroll
+            for (int off = kWave / 2; off > 0; off >>= 1) {
+                const float ov = __shfl_xor(best, off, kWave);
+                const int oe = __shfl_xor(best_e, off, kWave);
+                if (ov > best || (ov == best && oe < best_e)) {
+                    best = ov;
+                    best_e = oe;
+                }
+            }
+            const float sc = score_s[best_e];
+            chosen_sum += sc;
+            if (lane == 0) {
+                chosen[static_cast<size_t>(t) * top + c] = best_e;
+                weight[static_cast<size_t>(t) * top + c] = sc;
+            }
+            if (lane == best_e % kWave) z[best_e] = -INFINITY;
+        }
+        if (lane == 0) {
+            const float f = weight_scale / (chosen_sum + 1e-20f);
+            for (int c = 0; c < top; ++c) weight[static_cast<size_t>(t) * top + c] *= f;
+        }
+        return;
+    }
     // the top choices one after the other: the largest logit not yet taken, the lowest index among equals
     float first = 0.f, total = 0.f;
     for (int c = 0; c < top; ++c) {
@@ -219,6 +271,56 @@ __global__ __launch_bounds__(256) void moe_gate_up_kernel(const T* __restrict__ 
     }
 }
 
+// Experts without a gate: act = relu(x Wu^T)^2; w [experts][ff][hidden].  The same tiling with one product a wavefront.
+template <typename T, int RT>
+__global__ __launch_bounds__(256) void moe_up_kernel(const T* __restrict__ x, const T* __restrict__ w,
+                                                     const int32_t* __restrict__ row_token, const int32_t* __restrict__ tiles,
+                                                     T* __restrict__ act, int hidden, int ff) {
+    constexpr int E = 16 / sizeof(T);
+    if (static_cast<int>(blockIdx.x) >= tiles[0]) return;
+    const int32_t* tile = tiles + 1 + 3 * blockIdx.x;
+    const int expert = tile[0], row0 = tile[1], n_rows = tile[2];
+    const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+    const int lj = lane % 16, lg = lane / 16;
+    const int n0 = (blockIdx.y * (blockDim.x / kWave) + wave) * 16;
+    if (n0 >= ff) return;
+    const bool aligned = hidden % E == 0;
+    const T* wu = n0 + lj < ff ? w + (static_cast<size_t>(expert) * ff + n0 + lj) * hidden : nullptr;
+    const T* xr[RT];
+#pragma unroll
+    for (int r = 0; r < RT; ++r)
+        xr[r] = r * 16 + lj < n_rows ? x + static_cast<size_t>(row_token[row0 + r * 16 + lj]) * hidden : nullptr;
+    m_f32x4 u[RT];
+#pragma unroll
+    for (int r = 0; r < RT; ++r) u[r] = m_f32x4{0.f, 0.f, 0.f, 0.f};
+    constexpr int U = RT >= 4 ? 2 : 4;
+    for (int k0 = 0; k0 < hidden; k0 += 4 * E * U) {
+        m_u32x4 b[U], xv[U][RT];
+#pragma unroll
+        for (int s = 0; s < U; ++s) {
+            const int k = k0 + s * 4 * E + lg * E;
+            b[s] = row_piece<T>(wu, k, hidden, aligned);
+#pragma unroll
+            for (int r = 0; r < RT; ++r) xv[s][r] = row_piece<T>(xr[r], k, hidden, aligned);
+        }
+#pragma unroll
+        for (int s = 0; s < U; ++s)
+#pragma unroll
+            for (int r = 0; r < RT; ++r) u[r] = mma16<T>(b[s], xv[s][r], u[r]);
+    }
+#pragma unroll
+    for (int r = 0; r < RT; ++r) {
+        if (r * 16 + lj >= n_rows) continue;
+        T* o = act + static_cast<size_t>(row0 + r * 16 + lj) * ff;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int n = n0 + 4 * lg + v;
+            const float z = fmaxf(u[r][v], 0.f);
+            if (n < ff) o[n] = from_float<T>(z * z);
+        }
+    }
+}
+
 template <typename T, int RT>
 __global__ __launch_bounds__(256) void moe_down_kernel(const T* __restrict__ act, const T* __restrict__ w,
                                                        const int32_t* __restrict__ tiles, float* __restrict__ y, int hidden,
@@ -283,23 +385,24 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
 using namespace egpt;
 
 extern "C" int egpt_moe_route(const void* x, const void* router, const void* bias, int32_t* chosen, float* weight, int n_tokens,
-                              int hidden, int experts, int top, int dtype, void* stream) {
+                              int hidden, int experts, int top, int score_all, const float* correction, float weight_scale,
+                              int dtype, void* stream) {
     if (!x || !router || !chosen || !weight || n_tokens < 0 || hidden <= 0 || experts <= 0 || top <= 0 || top > experts ||
         (dtype != 0 && dtype != 1))
         return EGPT_BAD_ARGUMENT;
     if (experts > kMaxExperts) return EGPT_UNSUPPORTED_SIZE;
     if (n_tokens == 0) return EGPT_OK;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    const size_t lds = static_cast<size_t>(experts) * sizeof(float);
+    const size_t lds = 2 * static_cast<size_t>(experts) * sizeof(float);
     const unsigned blocks = n_tokens;
     if (dtype == 0)
         moe_route_kernel<float><<<blocks, 256, lds, s>>>(static_cast<const float*>(x), static_cast<const float*>(router),
                                                          static_cast<const float*>(bias), chosen, weight, n_tokens, hidden,
-                                                         experts, top);
+                                                         experts, top, score_all, correction, weight_scale);
     else
         moe_route_kernel<bf16_t><<<blocks, 256, lds, s>>>(static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(router),
                                                           static_cast<const bf16_t*>(bias), chosen, weight, n_tokens, hidden,
-                                                          experts, top);
+                                                          experts, top, score_all, correction, weight_scale);
     EGPT_CHECK_LAUNCH();
     return EGPT_OK;
 }
@@ -342,6 +445,30 @@ extern "C" int egpt_moe_gate_up(const void* x, const void* w_gate_up, const int3
         if (tile_rows == 16) EGPT_MOE_GU(bf16_t, 1); else if (tile_rows == 32) EGPT_MOE_GU(bf16_t, 2); else EGPT_MOE_GU(bf16_t, 4);
     }
 #undef EGPT_MOE_GU
+    EGPT_CHECK_LAUNCH();
+    return EGPT_OK;
+}
+
+extern "C" int egpt_moe_up(const void* x, const void* w_up, const int32_t* row_token, const int32_t* tiles, void* act, int n_rows,
+                           int hidden, int ff, int experts, int tile_rows, int dtype, void* stream) {
+    if (!x || !w_up || !row_token || !tiles || !act || n_rows < 0 || hidden <= 0 || ff <= 0 || experts <= 0 ||
+        (tile_rows != 16 && tile_rows != 32 && tile_rows != 64) || (dtype != 0 && dtype != 1))
+        return EGPT_BAD_ARGUMENT;
+    if (n_rows == 0) return EGPT_OK;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int max_tiles = n_rows / tile_rows + experts + 1;
+    const int nw = moe_waves(max_tiles, ff);
+    dim3 grid(max_tiles, (ff + nw * 16 - 1) / (nw * 16));
+    if (grid.y > 65535) return EGPT_UNSUPPORTED_SIZE;
+#define EGPT_MOE_UP(T_, RT_)                                                                                        \
+    moe_up_kernel<T_, RT_><<<grid, nw * 64, 0, s>>>(static_cast<const T_*>(x), static_cast<const T_*>(w_up), row_token, \
+                                                    tiles, static_cast<T_*>(act), hidden, ff)
+    if (dtype == 0) {
+        if (tile_rows == 16) EGPT_MOE_UP(float, 1); else if (tile_rows == 32) EGPT_MOE_UP(float, 2); else EGPT_MOE_UP(float, 4);
+    } else {
+        if (tile_rows == 16) EGPT_MOE_UP(bf16_t, 1); else if (tile_rows == 32) EGPT_MOE_UP(bf16_t, 2); else EGPT_MOE_UP(bf16_t, 4);
+    }
+#undef EGPT_MOE_UP
     EGPT_CHECK_LAUNCH();
     return EGPT_OK;
 }

@@ -97,6 +97,75 @@ __global__ __launch_bounds__(256) void normed_pair_mean_kernel(ProductView<T> a,
         out[base + j] = factor * (a_s[j] * inv_a * to_float(wa[j]) + b_s[j] * inv_b * to_float(wb[j]));
 }
 
+// x[t, :] = E[id_t, :] + P[position_t, :]: a token's vector plus a learned vector of its position, added in float32
+// and written as the float32 residual stream.
+template <typename T>
+__global__ __launch_bounds__(256) void embed_positions_kernel(const int32_t* __restrict__ ids, const int32_t* __restrict__ positions,
+                                                              const T* __restrict__ table, const T* __restrict__ pos_table,
+                                                              float* __restrict__ out, int hidden, int vocab, int max_pos) {
+    const int t = blockIdx.x;
+    int id = ids[t], p = positions[t];
+    id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);      // both are range-checked on the host; never read outside
+    p = p < 0 ? 0 : (p >= max_pos ? max_pos - 1 : p);
+    const T* row = table + static_cast<size_t>(id) * hidden;
+    const T* prow = pos_table + static_cast<size_t>(p) * hidden;
+    float* o = out + static_cast<size_t>(t) * hidden;
+    for (int j = threadIdx.x; j < hidden; j += blockDim.x) o[j] = to_float(row[j]) + to_float(prow[j]);
+}
+
+// A branch's output joins the stream behind a norm of its own:  x = h + mult * LN(y) * post_w  (LN without bias, the
+// statistics of y's row in two passes over LDS).  With a history (every earlier result of the depth, float32
+// [n_hist + 1][rows][hidden]) x is kept as result n_hist and what goes on is the weighted sum
+// v = sum_(j <= n_hist) mix[j] * hist[j]; otherwise v = x.  v is written to h_out (which may be h itself), and with a
+// next norm's weight LN(v) * next_w is written to `out` in the activation type.  One workgroup per row.
+template <typename T>
+__global__ __launch_bounds__(256) void post_norm_add_kernel(const float* h, ProductView<T> y,
+                                                            const T* __restrict__ post_w, float eps, float mult,
+                                                            float* hist, int n_hist, size_t hist_stride,
+                                                            const float* __restrict__ mix, float* h_out,
+                                                            const T* __restrict__ next_w, T* __restrict__ out, int hidden) {
+    extern __shared__ float row_s[];
+    __shared__ float scratch[16];
+    const size_t base = static_cast<size_t>(blockIdx.x) * hidden;
+    const float inv_n = 1.0f / static_cast<float>(hidden);
+    float sum = 0.f;
+    for (int j = threadIdx.x; j < hidden; j += blockDim.x) {
+        const float v = y.at(base + j);
+        row_s[j] = v;
+        sum += v;
+    }
+    float mean = block_sum(sum, scratch) * inv_n;
+    float dev = 0.f;
+    for (int j = threadIdx.x; j < hidden; j += blockDim.x) {
+        const float d = row_s[j] - mean;
+        dev = fmaf(d, d, dev);
+    }
+    float inv = 1.0f / sqrtf(block_sum(dev, scratch) * inv_n + eps);
+    sum = 0.f;
+    for (int j = threadIdx.x; j < hidden; j += blockDim.x) {
+        float x = h[base + j] + mult * ((row_s[j] - mean) * inv * to_float(post_w[j]));
+        if (hist != nullptr) {
+            hist[static_cast<size_t>(n_hist) * hist_stride + base + j] = x;
+            float v = 0.f;
+            for (int i = 0; i < n_hist; ++i) v = fmaf(mix[i], hist[static_cast<size_t>(i) * hist_stride + base + j], v);
+            x = fmaf(mix[n_hist], x, v);
+        }
+        h_out[base + j] = x;
+        row_s[j] = x;
+        sum += x;
+    }
+    if (next_w == nullptr) return;
+    mean = block_sum(sum, scratch) * inv_n;
+    dev = 0.f;
+    for (int j = threadIdx.x; j < hidden; j += blockDim.x) {
+        const float d = row_s[j] - mean;
+        dev = fmaf(d, d, dev);
+    }
+    inv = 1.0f / sqrtf(block_sum(dev, scratch) * inv_n + eps);
+    for (int j = threadIdx.x; j < hidden; j += blockDim.x)
+        out[base + j] = from_float<T>((row_s[j] - mean) * inv * to_float(next_w[j]));
+}
+
 __global__ __launch_bounds__(256) void tanh_cap_kernel(float* __restrict__ x, float cap, size_t n) {
     const float inv = 1.0f / cap;
     for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += static_cast<size_t>(gridDim.x) * blockDim.x)
@@ -160,6 +229,46 @@ extern "C" int egpt_normed_pair_mean(const void* a, int a_splits, const void* b,
         normed_pair_mean_kernel<bf16_t><<<n_rows, 256, lds, s>>>(
             stream_view<bf16_t>(a, a_splits, stride), stream_view<bf16_t>(b, b_splits, stride), static_cast<const bf16_t*>(bias_a),
             static_cast<const bf16_t*>(bias_b), static_cast<const bf16_t*>(wa), static_cast<const bf16_t*>(wb), eps, factor, out, hidden);
+    EGPT_CHECK_LAUNCH();
+    return EGPT_OK;
+}
+
+extern "C" int egpt_embed_positions(const int32_t* ids, const int32_t* positions, const void* table, const void* pos_table,
+                                    float* out, int n_tokens, int hidden, int vocab, int max_pos, int dtype, void* stream) {
+    if (!ids || !positions || !table || !pos_table || !out || n_tokens < 0 || hidden <= 0 || vocab <= 0 || max_pos <= 0 ||
+        (dtype != 0 && dtype != 1))
+        return EGPT_BAD_ARGUMENT;
+    if (n_tokens == 0) return EGPT_OK;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == 0)
+        embed_positions_kernel<float><<<n_tokens, 256, 0, s>>>(ids, positions, static_cast<const float*>(table),
+                                                               static_cast<const float*>(pos_table), out, hidden, vocab, max_pos);
+    else
+        embed_positions_kernel<bf16_t><<<n_tokens, 256, 0, s>>>(ids, positions, static_cast<const bf16_t*>(table),
+                                                                static_cast<const bf16_t*>(pos_table), out, hidden, vocab, max_pos);
+    EGPT_CHECK_LAUNCH();
+    return EGPT_OK;
+}
+
+extern "C" int egpt_post_norm_add(const float* h, const void* y, int y_splits, const void* post_w, float eps, float mult,
+                                  float* hist, int n_hist, const float* mix, float* h_out, const void* next_w, void* out,
+                                  int n_rows, int hidden, int dtype, void* stream) {
+    if (!h || !y || !post_w || !h_out || n_rows < 0 || hidden <= 0 || y_splits < 0 || n_hist < 0 || (dtype != 0 && dtype != 1))
+        return EGPT_BAD_ARGUMENT;
+    if ((hist != nullptr) != (mix != nullptr) || (next_w != nullptr) != (out != nullptr)) return EGPT_BAD_ARGUMENT;
+    if (hidden > 16384) return EGPT_UNSUPPORTED_SIZE;          // a row lies in LDS
+    if (n_rows == 0) return EGPT_OK;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const size_t stride = static_cast<size_t>(n_rows) * hidden;
+    const size_t lds = static_cast<size_t>(hidden) * sizeof(float);
+    if (dtype == 0)
+        post_norm_add_kernel<float><<<n_rows, 256, lds, s>>>(h, stream_view<float>(y, y_splits, stride),
+                                                             static_cast<const float*>(post_w), eps, mult, hist, n_hist, stride, mix,
+                                                             h_out, static_cast<const float*>(next_w), static_cast<float*>(out), hidden);
+    else
+        post_norm_add_kernel<bf16_t><<<n_rows, 256, lds, s>>>(h, stream_view<bf16_t>(y, y_splits, stride),
+                                                              static_cast<const bf16_t*>(post_w), eps, mult, hist, n_hist, stride, mix,
+                                                              h_out, static_cast<const bf16_t*>(next_w), static_cast<bf16_t*>(out), hidden);
     EGPT_CHECK_LAUNCH();
     return EGPT_OK;
 }

@@ -28,7 +28,7 @@ def _load_library() -> ctypes.CDLL:
         lib = ctypes.CDLL(path)
     except (build.BuildError, OSError) as e:
         raise KernelsUnavailable(f"the HIP kernel library could not be built or loaded: {e}") from e
-    if lib.egpt_abi_version() != 21:
+    if lib.egpt_abi_version() != 22:
         raise KernelsUnavailable(f"{path} has an unexpected ABI version")
     return lib
 
@@ -105,9 +105,14 @@ class HipKernels(KernelBackend):
             "egpt_head_norm_store": [vp, i, vp, i, i, f, vp, vp, vp, f, i, vp, vp, vp, i, i, i, i, i, i, i, vp],
             "egpt_latent_prep": [vp, i, vp, i, i, f, i, vp, vp, vp, f, vp, f, i, vp, vp, vp, i, i, i, i, i, i, i, vp],
             "egpt_sigmoid_gate": [vp, i, vp, i, vp, i, i, f, i, i, vp, i, i, i, vp],
-            "egpt_window_attention": [vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, i, f, i, i, vp, vp, i, i, vp],
+            "egpt_window_attention": [vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, i, f, i, i, vp, vp, i, i, vp, i, vp],
             "egpt_window_attention_tiled": [vp, vp, vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, i, f, i, i, vp, vp, i,
-                                            i, i, i, vp],
+                                            i, vp, i, i, i, vp],
+            "egpt_embed_positions": [vp, vp, vp, vp, vp, i, i, i, i, i, vp],
+            "egpt_post_norm_add": [vp, vp, i, vp, f, f, vp, i, vp, vp, vp, vp, i, i, i, vp],
+            "egpt_bounded_gate": [vp, i, i, i, vp, vp, vp, i, i, i, vp],
+            "egpt_ff_activation": [vp, i, i, i, i, vp, f, i, vp, i, i, vp],
+            "egpt_moe_up": [vp, vp, vp, vp, vp, i, i, i, i, i, i, vp],
             "egpt_embed_scaled": [vp, vp, f, vp, i, i, i, i, vp],
             "egpt_add_layernorm": [vp, vp, i, i, vp, vp, vp, f, vp, i, i, i, vp],
             "egpt_normed_pair_mean": [vp, i, vp, i, vp, vp, vp, vp, f, f, vp, i, i, i, vp],
@@ -115,8 +120,8 @@ class HipKernels(KernelBackend):
             "egpt_whole_norm_store": [vp, i, i, vp, vp, vp, vp, f, vp, f, i, vp, vp, vp, i, i, i, i, i, i, i, vp],
             "egpt_head_norm_gate": [vp, i, vp, f, vp, i, i, i, vp, i, i, i, i, vp],
             "egpt_channel_decay": [vp, i, i, i, i, vp, vp, f, vp, i, i, i, vp],
-            "egpt_decayed_state_scan": [vp, i, i, i, i, i, f, vp, vp, vp, vp, vp, vp, i, i, vp, i, i, i, i, vp],
-            "egpt_moe_route": [vp, vp, vp, vp, vp, i, i, i, i, i, vp],
+            "egpt_decayed_state_scan": [vp, i, i, i, i, i, f, vp, vp, vp, vp, vp, vp, i, i, vp, i, i, i, i, i, i, vp],
+            "egpt_moe_route": [vp, vp, vp, vp, vp, i, i, i, i, i, vp, f, i, vp],
             "egpt_moe_group": [vp, vp, vp, vp, vp, i, i, i, i, vp],
             "egpt_moe_gate_up": [vp, vp, vp, vp, vp, i, i, i, i, i, i, vp],
             "egpt_moe_down": [vp, vp, vp, vp, i, i, i, i, i, i, vp],
@@ -958,8 +963,15 @@ class HipKernels(KernelBackend):
                   out.data_ptr(), t, n, dt, self._stream())
 
     def window_attention(self, q, out, k_cache, v_cache, block_table, q_start, q_len, kv_len, nq, nkv, dk, dv, page_size,
-                         scale, window, keep_first, sink, max_q_len, max_kv_len, dist_bias=None):
+                         scale, window, keep_first, sink, max_q_len, max_kv_len, dist_bias=None, block=0, slopes=None):
         t = q.shape[0]
+        block = int(block or 0)
+        if block < 0:
+            raise ValueError(f"block ({block}) must not be negative")
+        if slopes is not None:
+            self._need(slopes, "slopes", _F32, (nq,))
+            if dist_bias is not None:
+                raise ValueError("the attention kernels take a bias table or slopes, not both")
         b, width = block_table.shape
         dt = self._act(q, "q")
         self._need(q, "q", None, (t, nq * dk))
@@ -980,7 +992,9 @@ class HipKernels(KernelBackend):
             raise ValueError(f"block table of width {width} cannot hold {max_kv_len} tokens at page size {page_size}")
         if dk > self.max_window_attention_dim or dv > self.max_window_attention_dim:
             raise ValueError(f"key size {dk} / value size {dv} is not supported (at most {self.max_window_attention_dim})")
-        shape = self._window_attention_shape(t, b, nq, nkv, dk, dv, page_size, window, keep_first, max_q_len, max_kv_len,
+        # (a block of positions bounds the keys that a row sees as a window of that many does)
+        reach = min(window, block) if window and block else (window or block)
+        shape = self._window_attention_shape(t, b, nq, nkv, dk, dv, page_size, reach, keep_first, max_q_len, max_kv_len,
                                              q.element_size())
         if shape is not None:
             row_tiles, n_splits = shape
@@ -991,14 +1005,14 @@ class HipKernels(KernelBackend):
             self._run("egpt_window_attention_tiled", q.data_ptr(), out.data_ptr(), self._ptr(part_o), self._ptr(part_ml),
                       k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(), width, q_start.data_ptr(),
                       q_len.data_ptr(), kv_len.data_ptr(), b, t, nq, nkv, dk, dv, page_size, float(scale), int(window),
-                      int(keep_first), self._ptr(sink), self._ptr(dist_bias), dist_far, n_splits, row_tiles, dt,
-                      self._stream())
+                      int(keep_first), self._ptr(sink), self._ptr(dist_bias), dist_far, block, self._ptr(slopes), n_splits,
+                      row_tiles, dt, self._stream())
             return
         # sizes that the matrix-core kernel does not take: the general kernel
         self._run("egpt_window_attention", q.data_ptr(), out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                   block_table.data_ptr(), width, q_start.data_ptr(), q_len.data_ptr(), kv_len.data_ptr(), b, t, nq, nkv,
                   dk, dv, page_size, float(scale), int(window), int(keep_first), self._ptr(sink), self._ptr(dist_bias),
-                  dist_far, dt, self._stream())
+                  dist_far, block, self._ptr(slopes), dt, self._stream())
 
 
     # ------------------------------------------------------------------ stream operations beyond the RMS norm
@@ -1045,6 +1059,62 @@ class HipKernels(KernelBackend):
                   self._stream())
         return out
 
+    def embed_positions(self, token_ids, positions, table, pos_table, out):
+        dt = self._act(table, "table")
+        v, h = table.shape
+        t = token_ids.shape[0]
+        self._need(token_ids, "token_ids", _I32, (t,))
+        self._need(positions, "positions", _I32, (t,))
+        self._need(table, "table")
+        self._need(pos_table, "pos_table", table.dtype, (pos_table.shape[0], h))
+        self._need(out, "out", _F32, (t, h))
+        self._run("egpt_embed_positions", token_ids.data_ptr(), positions.data_ptr(), table.data_ptr(), pos_table.data_ptr(),
+                  out.data_ptr(), t, h, v, int(pos_table.shape[0]), dt, self._stream())
+
+    def post_norm_add(self, h, y, post_weight, eps, mult, history=None, n_history=0, mix=None, next_weight=None, h_out=None):
+        """x = h + mult * LN(y) * post_weight, LN without bias over y's rows (y a product: act [T, H] or float32 partial
+        sums [S, T, H]).  With history (float32 [n, T, H], n > n_history) x is stored as history[n_history] and what goes on
+        is v = sum_(j <= n_history) mix[j] * history[j] (mix float32 [n_history + 1]); else v = x.  v is written to h_out
+        (h itself if None).  Returns LN(v) * next_weight as act [T, H], or None without next_weight."""
+        dt = self._act(post_weight, "post_weight")
+        t, hidden = h.shape
+        self._need(h, "h", _F32)
+        self._need(post_weight, "post_weight", None, (hidden,))
+        splits = self._product(y, "y", post_weight.dtype, t, hidden)
+        if history is not None:
+            self._need(history, "history", _F32)
+            if history.dim() != 3 or tuple(history.shape[1:]) != (t, hidden) or not 0 <= n_history < history.shape[0]:
+                raise ValueError(f"history must be [more than {n_history}, {t}, {hidden}], got {tuple(history.shape)}")
+            self._need(mix, "mix", _F32, (n_history + 1,))
+        h_out = h if h_out is None else h_out
+        self._need(h_out, "h_out", _F32, (t, hidden))
+        out = None
+        if next_weight is not None:
+            self._need(next_weight, "next_weight", post_weight.dtype, (hidden,))
+            out = torch.empty((t, hidden), dtype=post_weight.dtype, device=h.device)
+        self._run("egpt_post_norm_add", h.data_ptr(), y.data_ptr(), splits, post_weight.data_ptr(), float(eps), float(mult),
+                  self._ptr(history), int(n_history), self._ptr(mix) if history is not None else None, h_out.data_ptr(),
+                  self._ptr(next_weight), self._ptr(out), t, hidden, dt, self._stream())
+        return out
+
+    def ff_activation(self, z, cols, mode, out, coef=None, eps=0.0, gate_col=-1):
+        """out[t, j] = f(z[t, j]) for j < cols of a product z (act [T, W] or float32 partial sums [S, T, W]): mode
+        'relu2' relu(z)^2; 'polynorm' coef[0] N(z) + coef[1] N(z^2) + coef[2] N(z^3) + coef[3], N(u) = u / sqrt(mean(u^2)
+        + eps) over the row's cols values (coef float32 [4]); gate_col >= 0: times sigmoid(z[t, gate_col])."""
+        t, width = z.shape[-2], z.shape[-1]
+        dt = self._act(out, "out")
+        self._need(out, "out", None, (t, cols))
+        splits = self._product(z, "z", out.dtype, t, width)
+        modes = {"relu2": 0, "polynorm": 1}
+        if mode not in modes:
+            raise ValueError(f"unknown activation '{mode}' (relu2, polynorm)")
+        if mode == "polynorm":
+            self._need(coef, "coef", _F32, (4,))
+        if not 0 < cols <= width or not -1 <= gate_col < width:
+            raise ValueError(f"{cols} columns and gate column {gate_col} do not fit rows of {width} values")
+        self._run("egpt_ff_activation", z.data_ptr(), splits, int(width), int(cols), modes[mode],
+                  self._ptr(coef) if mode == "polynorm" else None, float(eps), int(gate_col), out.data_ptr(), t, dt, self._stream())
+
     def tanh_cap(self, x, cap):
         self._need(x, "x", _F32)
         self._run("egpt_tanh_cap", x.data_ptr(), float(cap), x.numel(), self._stream())
@@ -1066,6 +1136,8 @@ class HipKernels(KernelBackend):
             self._need(k_weight, "k_weight", q_out.dtype, (nkv * dk,))
         if every:
             self._need(positions, "positions", _I32, (t,))
+        if nkv == 0 and slots is not None:
+            raise ValueError("rows of queries alone (nkv 0) have nothing to store")
         if slots is not None:
             self._need(slots, "slots", _I32, (t,))
             self._key_value_pages(k_cache, v_cache, q_out.dtype, nkv, page_size, dk, dv)
@@ -1080,11 +1152,13 @@ class HipKernels(KernelBackend):
         x_splits = self._product(x, "x", _F32, t, heads * dv)
         self._need(out, "out", None, (t, heads * dv))
         self._need(weight, "weight", out.dtype, (dv,))
-        width = gate.shape[-1]
-        splits = self._product(gate, "gate", out.dtype, t, width)
-        if gate_offset < 0 or gate_offset + heads * dv > width:
-            raise ValueError(f"gate columns {gate_offset}..{gate_offset + heads * dv} lie outside rows of {width} values")
-        self._run("egpt_head_norm_gate", x.data_ptr(), x_splits, weight.data_ptr(), float(eps), gate.data_ptr(), splits, int(width),
+        width, splits = 0, 0
+        if gate is not None:
+            width = gate.shape[-1]
+            splits = self._product(gate, "gate", out.dtype, t, width)
+            if gate_offset < 0 or gate_offset + heads * dv > width:
+                raise ValueError(f"gate columns {gate_offset}..{gate_offset + heads * dv} lie outside rows of {width} values")
+        self._run("egpt_head_norm_gate", x.data_ptr(), x_splits, weight.data_ptr(), float(eps), self._ptr(gate), splits, int(width),
                   int(gate_offset), out.data_ptr(), t, heads, dv, dt, self._stream())
 
     # ------------------------------------------------------------------ a decaying matrix state per head
@@ -1103,8 +1177,26 @@ class HipKernels(KernelBackend):
                   self._ptr(bias), float(tau), out.data_ptr(), t, channels, dt, self._stream())
         return out
 
+    def bounded_gate(self, z, z_offset, channels, bias, lower):
+        """float32 [T, channels]: lower + (1 - lower) * sigmoid(z[:, z_offset : z_offset + channels] + bias)."""
+        t, width = z.shape[-2], z.shape[-1]
+        ref = bias if bias is not None else lower
+        if ref is None:
+            raise ValueError("a bounded gate needs a bias or a lower bound (its type is the product's)")
+        dt = self._act(ref, "bias")
+        for name, v in (("bias", bias), ("lower", lower)):
+            if v is not None:
+                self._need(v, name, ref.dtype, (channels,))
+        splits = self._product(z, "z", ref.dtype, t, width)
+        if z_offset < 0 or z_offset + channels > width:
+            raise ValueError(f"columns {z_offset}..{z_offset + channels} lie outside rows of {width} values")
+        out = torch.empty((t, channels), dtype=_F32, device=ref.device)
+        self._run("egpt_bounded_gate", z.data_ptr(), splits, int(width), int(z_offset), self._ptr(bias), self._ptr(lower),
+                  out.data_ptr(), t, int(channels), dt, self._stream())
+        return out
+
     def decayed_state_scan(self, proj, act_dtype, q_offset, k_offset, v_offset, q_scale, decay, states, slots, fresh, q_start,
-                           q_len, heads, dk, dv):
+                           q_len, heads, dk, dv, q_silu=False, tied_keys=False):
         t, width = proj.shape[-2], proj.shape[-1]
         if act_dtype not in _DT:
             raise TypeError("act_dtype must be float32 or bfloat16")
@@ -1119,13 +1211,14 @@ class HipKernels(KernelBackend):
         self._need(q_len, "q_len", _I32, (b,))
         if fresh is not None:
             self._need(fresh, "fresh", torch.bool, (b,))
-        for off, n in ((q_offset, heads * dk), (k_offset, heads * dk), (v_offset, heads * dv)):
-            if off < 0 or off + n > width:
+        for off, n in ((q_offset, heads * dk), (None if tied_keys else k_offset, heads * dk), (v_offset, heads * dv)):
+            if off is not None and (off < 0 or off + n > width):
                 raise ValueError(f"columns {off}..{off + n} lie outside rows of {width} values")
         out = torch.empty((self.lib.egpt_scan_key_splits(dk), t, heads * dv), dtype=_F32, device=decay.device)
-        self._run("egpt_decayed_state_scan", proj.data_ptr(), splits, int(width), int(q_offset), int(k_offset), int(v_offset),
+        self._run("egpt_decayed_state_scan", proj.data_ptr(), splits, int(width), int(q_offset), 0 if tied_keys else int(k_offset), int(v_offset),
                   float(q_scale), decay.data_ptr(), states.data_ptr(), slots.data_ptr(), self._ptr(fresh), q_start.data_ptr(),
-                  q_len.data_ptr(), b, t, out.data_ptr(), heads, dk, dv, _DT[act_dtype], self._stream())
+                  q_len.data_ptr(), b, t, out.data_ptr(), heads, dk, dv, int(bool(q_silu)), int(bool(tied_keys)),
+                  _DT[act_dtype], self._stream())
         return out
 
     # ------------------------------------------------------------------ a mixture of experts
@@ -1135,19 +1228,24 @@ class HipKernels(KernelBackend):
         per_expert = n_rows / max(experts, 1)
         return 16 if per_expert <= 24 else (32 if per_expert <= 96 else 64)
 
-    def expert_mixture(self, x, router, router_bias, w_gate_up, w_down, top):
+    def expert_mixture(self, x, router, router_bias, w_gate_up, w_down, top, gated=True, score_all=False, correction=None,
+                       weight_scale=1.0):
         """float32 [T, H]: for every token the `top` experts with the largest float32 router logits (x router^T + bias),
         weighted by the softmax over those logits; an expert is down(silu(gate x) * (up x)).  w_gate_up [E, 2 ff, H]
-        (an expert's gate rows, then its up rows), w_down [E, H, ff]."""
+        (an expert's gate rows, then its up rows), w_down [E, H, ff].  gated False: an expert is down(relu(up x)^2) and
+        w_gate_up is [E, ff, H].  score_all: the scores are the softmax over all experts, the choice goes by score +
+        correction (float32 [E] or None), the weights are the chosen scores over their sum, times weight_scale."""
         t, hidden = x.shape
         dt = self._act(x, "x")
         experts, ff2, _ = w_gate_up.shape
-        ff = ff2 // 2
+        ff = ff2 // 2 if gated else ff2
+        if correction is not None:
+            self._need(correction, "correction", _F32, (experts,))
         self._need(x, "x")
         self._need(router, "router", x.dtype, (experts, hidden))
         if router_bias is not None:
             self._need(router_bias, "router_bias", x.dtype, (experts,))
-        self._need(w_gate_up, "w_gate_up", x.dtype, (experts, 2 * ff, hidden))
+        self._need(w_gate_up, "w_gate_up", x.dtype, (experts, 2 * ff if gated else ff, hidden))
         self._need(w_down, "w_down", x.dtype, (experts, hidden, ff))
         if not 0 < top <= experts:
             raise ValueError(f"top ({top}) must be between 1 and the number of experts ({experts})")
@@ -1167,11 +1265,11 @@ class HipKernels(KernelBackend):
         out = torch.empty((t, hidden), dtype=_F32, device=dev)
         st = self._stream()
         self._run("egpt_moe_route", x.data_ptr(), router.data_ptr(), self._ptr(router_bias), chosen.data_ptr(),
-                  weight.data_ptr(), t, hidden, experts, top, dt, st)
+                  weight.data_ptr(), t, hidden, experts, top, int(bool(score_all)), self._ptr(correction), float(weight_scale), dt, st)
         self._run("egpt_moe_group", chosen.data_ptr(), row_token.data_ptr(), place.data_ptr(), tiles.data_ptr(),
                   counts.data_ptr(), t, top, experts, tile_rows, st)
-        self._run("egpt_moe_gate_up", x.data_ptr(), w_gate_up.data_ptr(), row_token.data_ptr(), tiles.data_ptr(),
-                  act.data_ptr(), n_rows, hidden, ff, experts, tile_rows, dt, st)
+        self._run("egpt_moe_gate_up" if gated else "egpt_moe_up", x.data_ptr(), w_gate_up.data_ptr(), row_token.data_ptr(),
+                  tiles.data_ptr(), act.data_ptr(), n_rows, hidden, ff, experts, tile_rows, dt, st)
         self._run("egpt_moe_down", act.data_ptr(), w_down.data_ptr(), tiles.data_ptr(), y.data_ptr(), n_rows, hidden, ff,
                   experts, tile_rows, dt, st)
         self._run("egpt_moe_combine", y.data_ptr(), place.data_ptr(), weight.data_ptr(), out.data_ptr(), t, top, hidden, st)

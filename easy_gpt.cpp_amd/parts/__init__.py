@@ -1,4 +1,5 @@
-from . import attention, block, branch_mixers, embedding, expert_mixture, feed_forward, head_attention, norm, position  # noqa: F401  (register the built-in parts)
+from . import (attention, block, branch_mixers, depth_average, embedding, expert_mixture, feed_forward, gated_recurrence,  # noqa: F401
+               head_attention, local_attention, norm, position)      # (register the built-in parts)
 from .base import (
     BLOCKS,
     FEED_FORWARDS,
@@ -19,6 +20,7 @@ from .base import (
     PositionEncoding,
     StateNeed,
     StateView,
+    StreamJoin,
     make_part,
     register_part,
 )
@@ -28,6 +30,6 @@ from .spec import LayerSpec, ModelSpec, ParamSpec, PartSpec, RunSpec
 __all__ = [
     "BLOCKS", "FEED_FORWARDS", "MIXERS", "NORMS", "POSITION_ENCODINGS", "Block", "CacheGroup", "CacheNeed",
     "CacheView", "Embedding", "FeedForward", "LayerSpec", "Mixer", "Model", "ModelSpec", "Norm", "OutputHead", "PagedTensor", "ParamSpec", "Part",
-    "PartSpec", "PendingNorm", "PositionEncoding", "RunSpec", "StateNeed", "StateView", "build_model", "make_part",
+    "PartSpec", "PendingNorm", "PositionEncoding", "RunSpec", "StateNeed", "StateView", "StreamJoin", "build_model", "make_part",
     "register_part",
 ]

@@ -271,6 +271,12 @@ class OutputHead(Part):
         raise NotImplementedError
 
 
+class StreamJoin(Part):
+    """Decides what the next layer reads once a layer's own result is known.  An arrangement that takes one
+    (`Block.takes_stream_join`) hands it the step's context and calls what the join offers; the one built-in kind keeps
+    every result of the depth and goes on with a learned weighted sum of them (`parts/depth_average.py`)."""
+
+
 class Block:
     """Arrangement of one layer's parts around the residual stream.
 
@@ -286,6 +292,7 @@ class Block:
     norm_slots: tuple[str, ...] = ()     # names of the norms this arrangement places
     uses_mixer = True
     uses_feed_forward = True
+    takes_stream_join = False            # True: the constructor takes `stream_join=` (a StreamJoin or None)
 
     def __init__(self, mixer: Mixer | None, feed_forward: FeedForward | None, norms: dict[str, Norm]):
         if set(norms) != set(self.norm_slots):
@@ -312,6 +319,7 @@ POSITION_ENCODINGS: dict[str, Callable[..., PositionEncoding]] = {}
 BLOCKS: dict[str, Callable[..., Block]] = {}
 EMBEDDINGS: dict[str, Callable[..., Part]] = {}
 OUTPUT_HEADS: dict[str, Callable[..., Part]] = {}
+STREAM_JOINS: dict[str, Callable[..., StreamJoin]] = {}
 
 _REGISTRIES = {
     "mixer": MIXERS,
@@ -321,12 +329,13 @@ _REGISTRIES = {
     "block": BLOCKS,
     "embedding": EMBEDDINGS,
     "output_head": OUTPUT_HEADS,
+    "stream_join": STREAM_JOINS,
 }
 
 
 def register_part(family: str, kind: str, factory: Callable[..., Any], replace: bool = False) -> None:
     """Add a part under `kind` to one of the families: mixer, feed_forward, norm,
-    position_encoding, block, embedding, output_head."""
+    position_encoding, block, embedding, output_head, stream_join."""
     reg = _REGISTRIES[family]
     if kind in reg and not replace:
         raise ValueError(f"{family} '{kind}' is already registered")

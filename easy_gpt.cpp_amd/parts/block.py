@@ -103,3 +103,68 @@ register_part("block", "pre_norm", PreNormBlock)
 register_part("block", "pre_norm_mixer_only", PreNormMixerOnlyBlock)
 register_part("block", "parallel", ParallelBlock)
 register_part("block", "parallel_mixer_only", ParallelMixerOnlyBlock)
+
+
+class SandwichBlock(Block):
+    """A norm before and a norm behind each branch, and a constant factor on what a branch adds:
+    a = h + m * N1b(Mixer(N1(h))); y = a + m * N2b(FF(N2(a))).  The norms behind the branches read the branches' products
+    unrounded (float32 partial sums) and the additions are float32, in one kernel with the norm that follows them where
+    there is one.  With a stream join that keeps the depth's results (`parts/depth_average.py`), y is stored among them
+    and what the next layer reads is their weighted sum, written by the kernel of the layer's last addition.  The norms
+    are the layer norm without bias (`layernorm`, whose weight and eps the fused kernel takes)."""
+
+    norm_slots = ("mixer", "mixer_out", "feed_forward", "feed_forward_out")
+    takes_stream_join = True
+
+    def __init__(self, mixer, feed_forward, norms, residual_mult: float = 1.0, stream_join=None):
+        super().__init__(mixer, feed_forward, norms)
+        self.residual_mult = float(residual_mult)
+        self.stream_join = stream_join
+        for slot in self.norm_slots:
+            n = self.norms[slot]
+            if getattr(n, "bias_name", "") is not None or not hasattr(n, "eps"):
+                raise ValueError(f"the sandwich arrangement's norm '{slot}' must be a layer norm without bias")
+
+    def parts(self):
+        return super().parts() + ([self.stream_join] if self.stream_join is not None else [])
+
+    def _last_addition(self, h, y, norm, ctx):
+        """h + m * norm(y), through the stream join if there is one: the stream that goes on."""
+        k = kernels.backend()
+        join = self.stream_join
+        if join is None:
+            k.post_norm_add(h, y, norm.weight, norm.eps, self.residual_mult)
+            return h
+        kept = join.results(ctx, h)
+        k.post_norm_add(h, y, norm.weight, norm.eps, self.residual_mult, history=kept, n_history=join.index, mix=join.weights)
+        return h
+
+    def forward(self, h, delta, ctx, cache, state):
+        if h.dtype != torch.float32:
+            raise TypeError("the sandwich arrangement keeps its stream in float32")
+        k = kernels.backend()
+        if self.stream_join is not None:
+            self.stream_join.results(ctx, h)                              # (the first layer keeps the embedding's output)
+        x = self.norms["mixer"].forward(h, delta)                         # adds what is pending, if anything
+        y = self.mixer.forward(x, ctx, cache, state)
+        if self.feed_forward is None:
+            return self._last_addition(h, y, self.norms["mixer_out"], ctx), None
+        post, pre = self.norms["mixer_out"], self.norms["feed_forward"]
+        if pre.eps == post.eps:
+            x = k.post_norm_add(h, y, post.weight, post.eps, self.residual_mult, next_weight=pre.weight)
+        else:
+            k.post_norm_add(h, y, post.weight, post.eps, self.residual_mult)
+            x = pre.forward(h, None)
+        z = self.feed_forward.forward(x, ctx)
+        return self._last_addition(h, z, self.norms["feed_forward_out"], ctx), None
+
+
+class SandwichMixerOnlyBlock(SandwichBlock):
+    """The sandwich arrangement of a layer that has no feed-forward: y = h + m * N1b(Mixer(N1(h)))."""
+
+    norm_slots = ("mixer", "mixer_out")
+    uses_feed_forward = False
+
+
+register_part("block", "sandwich", SandwichBlock)
+register_part("block", "sandwich_mixer_only", SandwichMixerOnlyBlock)

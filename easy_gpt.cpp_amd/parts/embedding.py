@@ -87,6 +87,33 @@ class ScaledTokenEmbedding(TokenEmbedding):
         return out
 
 
+class PositionedTokenEmbedding(TokenEmbedding):
+    """x[t, :] = E[id_t, :] + P[position_t, :] with a learned vector per position (the tensor `prefix + position_name`,
+    [max_positions, H]), added in float32 and written as a float32 residual stream.  A request cannot grow beyond the
+    table's rows (the model's `max_position`)."""
+
+    def __init__(self, prefix: str, hidden_size: int, vocab_size: int, max_positions: int, name: str = "weight",
+                 position_name: str = "pos"):
+        super().__init__(prefix, hidden_size, vocab_size, name)
+        self.max_positions = int(max_positions)
+        self.position_name = position_name
+        self.position_table: torch.Tensor | None = None
+
+    def param_specs(self):
+        return super().param_specs() + [ParamSpec(self.prefix + self.position_name, (self.max_positions, self.hidden_size),
+                                                  role="embedding")]
+
+    def load(self, get, dtype, device):
+        super().load(get, dtype, device)
+        self.position_table = self._to(get(self.prefix + self.position_name), "compute", dtype, device)
+
+    def forward(self, ctx) -> torch.Tensor:
+        token_ids = ctx.token_ids
+        out = torch.empty((token_ids.shape[0], self.hidden_size), device=token_ids.device, dtype=torch.float32)
+        kernels.backend().embed_positions(token_ids, ctx.positions, self.table, self.position_table, out)
+        return out
+
+
 class LinearHead(OutputHead):
     graph_safe = True
 
@@ -127,4 +154,5 @@ class LinearHead(OutputHead):
 register_part("embedding", "token_embedding", TokenEmbedding)
 register_part("embedding", "token_embedding_normed", NormedTokenEmbedding)
 register_part("embedding", "token_embedding_scaled", ScaledTokenEmbedding)
+register_part("embedding", "token_embedding_positions", PositionedTokenEmbedding)
 register_part("output_head", "linear_head", LinearHead)

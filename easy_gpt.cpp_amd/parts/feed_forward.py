@@ -88,4 +88,57 @@ class SwiGLU(FeedForward):
         return down(act)
 
 
+class ActivatedFeedForward(FeedForward):
+    """A feed-forward without a gate product: y = W_down act(W_up x), no biases.
+
+    activation 'relu2': the square of relu.  'polynorm': c0 N(z) + c1 N(z^2) + c2 N(z^3) + c3 with powers taken element
+    by element, N(u) = u / sqrt(mean(u^2) + eps) over a token's inner values, and the four numbers c in the tensor
+    `coef`.  row_gate: the name of a [1, H] tensor g; the token's output is multiplied by sigmoid(g . x), one number
+    per token (its weights ride as one more row of the up matrix, and since the down product is linear the factor is
+    applied to the activated inner values).  The up product stays unrounded (float32) until the activation has used it;
+    the statistics and the activation are float32.  The output is float32 partial sums."""
+
+    graph_safe = True
+
+    def __init__(self, prefix: str, hidden_size: int, intermediate_size: int, activation: str = "relu2", eps: float = 0.0,
+                 names: tuple[str, str] = ("up", "down"), coef: str = "act", row_gate: str | None = None):
+        if activation not in ("relu2", "polynorm"):
+            raise ValueError(f"activation '{activation}' is not supported by this feed-forward (relu2, polynorm)")
+        self.prefix, self.hidden_size, self.intermediate_size = prefix, int(hidden_size), int(intermediate_size)
+        self.activation, self.eps = activation, float(eps)
+        self.names, self.coef_name, self.row_gate = tuple(names), coef, row_gate
+        self.w_up = self.w_down = self.coef = None
+
+    def param_specs(self):
+        p, h, i = self.prefix, self.hidden_size, self.intermediate_size
+        up, down = self.names
+        specs = [ParamSpec(p + up, (i, h)), ParamSpec(p + down, (h, i))]
+        if self.activation == "polynorm":
+            specs.append(ParamSpec(p + self.coef_name, (4,), role="norm_scale", dtype="float32"))
+        if self.row_gate is not None:
+            specs.append(ParamSpec(p + self.row_gate, (1, h), alt_shapes=((h,),)))
+        return specs
+
+    def load(self, get, dtype, device):
+        p = self.prefix
+        up, down = self.names
+        rows = [get(p + up).to(dtype)]
+        if self.row_gate is not None:
+            rows.append(get(p + self.row_gate).to(dtype).reshape(1, self.hidden_size))
+        self.w_up = torch.cat(rows, dim=0).to(device).contiguous()
+        self.w_down = self._to(get(p + down), "compute", dtype, device)
+        if self.activation == "polynorm":
+            self.coef = get(p + self.coef_name).to(torch.float32).reshape(4).to(device).contiguous()
+
+    def forward(self, x, ctx=None):
+        k = kernels.backend()
+        i = self.intermediate_size
+        z = k.product(x, self.w_up, unrounded=True)
+        act = torch.empty((x.shape[0], i), dtype=x.dtype, device=x.device)
+        k.ff_activation(z, i, self.activation, act, coef=self.coef, eps=self.eps, gate_col=i if self.row_gate is not None else -1)
+        out = k.product(act, self.w_down, unrounded=True)
+        return out if out.dim() == 3 else out.float()[None]
+
+
 register_part("feed_forward", "swiglu", SwiGLU)
+register_part("feed_forward", "activated", ActivatedFeedForward)

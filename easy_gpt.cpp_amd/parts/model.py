@@ -36,7 +36,12 @@ class Model:
             mixer = make_part("mixer", ls.mixer, **ctx) if ls.mixer is not None else None
             ff = make_part("feed_forward", ls.feed_forward, **ctx) if ls.feed_forward is not None else None
             norms = {slot: make_part("norm", ns, **ctx) for slot, ns in ls.norms.items()}
-            self.layers.append(BLOCKS[ls.block](mixer, ff, norms))
+            extra = dict(ls.block_params)
+            if ls.stream_join is not None:
+                if not getattr(BLOCKS[ls.block], "takes_stream_join", False):
+                    raise ValueError(f"the block arrangement '{ls.block}' takes no stream join")
+                extra["stream_join"] = make_part("stream_join", ls.stream_join, **ctx)
+            self.layers.append(BLOCKS[ls.block](mixer, ff, norms, **extra))
         self.final_norm = make_part("norm", spec.final_norm, **ctx)
         self.output_head = make_part("output_head", spec.output_head, vocab_size=spec.vocab_size, **ctx)
         self.dtype: torch.dtype | None = None

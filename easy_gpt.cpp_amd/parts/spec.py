@@ -15,7 +15,7 @@ class ParamSpec:
     """One tensor of the weights file.
 
     role    how random weights draw it: 'matrix', 'embedding', 'bias' ~ N(0, 0.02);
-            'norm_scale' ~ 1 + N(0, 0.02); 'int_table' uniform integers; or any role that was added
+            'norm_scale' ~ 1 + N(0, 0.02); 'mean_weights' ~ (1 + N(0, 0.02)) / n; 'int_table' uniform integers; or any role that was added
             with `weights.register_role` (a decay in (0, 1), a table of a special form, ...)
     dtype   'compute' (cast to the engine's dtype), 'float32' or 'int32' (kept as stored)
     alt_shapes  other shapes accepted on load (the reference accepts [H, 1] for a
@@ -50,12 +50,18 @@ class LayerSpec:
             'mixer' and 'feed_forward' for the pre-norm block; an arrangement with norms before and after each
             branch declares four, one with a single shared norm one)
     mixer, feed_forward   None where the arrangement has no such part (`Block.uses_mixer`, `uses_feed_forward`)
+    block_params   constants of the arrangement itself (a factor on what its branches add to the stream, say), passed
+            to the arrangement's constructor by name
+    stream_join   a part of the family 'stream_join' that decides what goes on to the next layer once the layer's own
+            result is known (a weighted sum over the results of all layers so far, say); None: the result itself
     """
 
     block: str
     mixer: PartSpec | None
     feed_forward: PartSpec | None
     norms: Mapping[str, PartSpec] = field(default_factory=dict)
+    block_params: Mapping[str, Any] = field(default_factory=dict)
+    stream_join: PartSpec | None = None
 
 
 @dataclass(frozen=True)

@@ -1,7 +1,7 @@
 """Random-weights mode: a model folder (config.json, model.safetensors) from a configuration and a seed.
 
 Distributions by a tensor's role (`ParamSpec.role`): matrices, embeddings and biases ~ N(0, 0.02); norm scales
-~ 1 + N(0, 0.02); integer tables uniform.  `register_role` adds a role with a distribution of its own.
+~ 1 + N(0, 0.02); the n weights of a weighted sum ~ (1 + N(0, 0.02)) / n; integer tables uniform.  `register_role` adds a role with a distribution of its own.
 Each tensor has a key made of (seed, tensor name), and element i of it is a function of (key, i) alone, computed
 with integer operations: the values do not depend on the order in which tensors are made nor on the device that
 draws them (a GPU draws a large model's tensors in seconds, the CPU draws the same ones).  The normal distribution is
@@ -96,6 +96,14 @@ def _norm_scale(shape, g, device):
     return _counter_normal(shape, g.initial_seed(), device, _STD, 1.0)
 
 
+def _mean_weights(shape, g, device):
+    """The weights of a weighted sum of n terms: (1 + N(0, 0.02)) / n, so that the sum keeps the size of its terms."""
+    n = 1
+    for d in shape:
+        n *= int(d)
+    return _counter_normal(shape, g.initial_seed(), device, _STD / max(n, 1), 1.0 / max(n, 1))
+
+
 def _int_table(shape, g, device):
     n = 1
     for d in shape:
@@ -111,6 +119,7 @@ ROLES: dict[str, Callable[..., torch.Tensor]] = {
     "embedding": _normal,
     "bias": _normal,
     "norm_scale": _norm_scale,
+    "mean_weights": _mean_weights,
     "int_table": _int_table,
 }
 
