@@ -177,7 +177,7 @@ class EmulatedKernels(KernelBackend):
         out.copy_((xx * torch.sigmoid(g)).to(out.dtype))
 
     def window_attention(self, q, out, k_cache, v_cache, block_table, q_start, q_len, kv_len, nq, nkv, dk, dv, page_size,
-                         scale, window, keep_first, sink, max_q_len, max_kv_len, dist_bias=None):
+                         scale, window, keep_first, sink, max_q_len, max_kv_len, dist_bias=None, block=0, slopes=None):
         group = nq // nkv
         q_all = q.view(q.shape[0], nq, dk).to(F64)
         for b in range(q_start.shape[0]):
@@ -185,6 +185,8 @@ class EmulatedKernels(KernelBackend):
             for i in range(n):
                 p = kv - n + i
                 lo = max(0, p - window + 1) if window else 0
+                if block:
+                    lo = max(lo, p // block * block)
                 js = torch.cat([torch.arange(0, min(keep_first, lo)), torch.arange(lo, p + 1)])
                 pages = block_table[b, (js // page_size)].long()
                 assert (pages >= 0).all(), "attention would read a page that was given back"
@@ -196,6 +198,8 @@ class EmulatedKernels(KernelBackend):
                     sc = (keys @ q_all[s + i, h]) * scale
                     if dist_bias is not None:
                         sc = sc + dist_bias[h, (p - js).clamp(max=dist_bias.shape[1] - 1)].to(F64)
+                    if slopes is not None:
+                        sc = sc - slopes[h].to(F64) * (p - js).to(F64)
                     m = sc.max() if sink is None else torch.maximum(sc.max(), sink[h].to(F64))
                     e = torch.exp(sc - m)
                     denom = e.sum() + (torch.exp(sink[h].to(F64) - m) if sink is not None else 0.0)
@@ -253,6 +257,9 @@ class EmulatedKernels(KernelBackend):
         t = out.shape[0]
         xx = _whole(x).to(F64).view(t, heads, dv)
         xx = xx / torch.sqrt((xx * xx).mean(-1, keepdim=True) + eps) * weight.to(F64)
+        if gate is None:
+            out.copy_(xx.reshape(t, heads * dv).to(out.dtype))
+            return
         g = _whole(gate)[:, gate_offset : gate_offset + heads * dv].to(F64)
         out.copy_((xx.reshape(t, heads * dv) * g * torch.sigmoid(g)).to(out.dtype))
 
@@ -262,8 +269,15 @@ class EmulatedKernels(KernelBackend):
             z = z + bias.to(F64)
         return (torch.sigmoid(z) ** (1.0 / tau)).to(torch.float32)
 
+    def bounded_gate(self, z, z_offset, channels, bias, lower):
+        v = _whole(z)[:, z_offset : z_offset + channels].to(F64)
+        if bias is not None:
+            v = v + bias.to(F64)
+        low = lower.to(F64) if lower is not None else 0.0
+        return (low + (1.0 - low) * torch.sigmoid(v)).to(torch.float32)
+
     def decayed_state_scan(self, proj, act_dtype, q_offset, k_offset, v_offset, q_scale, decay, states, slots, fresh, q_start,
-                           q_len, heads, dk, dv):
+                           q_len, heads, dk, dv, q_silu=False, tied_keys=False):
         x = _whole(proj).to(F64)
         t = x.shape[0]
         out = torch.zeros((t, heads * dv), dtype=torch.float32)
@@ -273,30 +287,72 @@ class EmulatedKernels(KernelBackend):
                 continue
             st = torch.zeros((heads, dk, dv), dtype=F64) if fresh is not None and bool(fresh[b]) else states[slot].to(F64)
             for i in range(s0, s0 + n):
-                q = x[i, q_offset : q_offset + heads * dk].view(heads, dk) * q_scale
-                k = x[i, k_offset : k_offset + heads * dk].view(heads, dk)
+                q = x[i, q_offset : q_offset + heads * dk].view(heads, dk)
+                q = (q * torch.sigmoid(q) if q_silu else q) * q_scale
+                k = 1.0 - decay[i].to(F64).view(heads, dk) if tied_keys else x[i, k_offset : k_offset + heads * dk].view(heads, dk)
                 v = x[i, v_offset : v_offset + heads * dv].view(heads, dv)
                 st = decay[i].to(F64).view(heads, dk)[:, :, None] * st + k[:, :, None] * v[:, None, :]
                 out[i] = torch.einsum("hkv,hk->hv", st, q).reshape(-1).to(torch.float32)
             states[slot] = st.to(states.dtype)
         return out
 
-    def expert_mixture(self, x, router, router_bias, w_gate_up, w_down, top):
+    def expert_mixture(self, x, router, router_bias, w_gate_up, w_down, top, gated=True, score_all=False, correction=None,
+                       weight_scale=1.0):
         xx = x.to(F64)
         z = xx @ router.to(F64).T
         if router_bias is not None:
             z = z + router_bias.to(F64)
-        val, idx = torch.topk(z, top, dim=-1)
-        wt = torch.softmax(val, dim=-1)
-        ff = w_gate_up.shape[1] // 2
+        if score_all:
+            sc = torch.softmax(z, dim=-1)
+            pick = sc if correction is None else sc + correction.to(F64)
+            idx = torch.argsort(-pick, dim=-1, stable=True)[:, :top]
+            val = torch.gather(sc, -1, idx)
+            wt = val / (val.sum(-1, keepdim=True) + 1e-20) * weight_scale
+        else:
+            val, idx = torch.topk(z, top, dim=-1)
+            wt = torch.softmax(val, dim=-1)
+        ff = w_gate_up.shape[1] // 2 if gated else w_gate_up.shape[1]
         out = torch.zeros(x.shape, dtype=F64)
         for t in range(x.shape[0]):
             for c in range(top):
                 e = int(idx[t, c])
                 gu = w_gate_up[e].to(F64) @ xx[t]
-                act = (gu[:ff] * torch.sigmoid(gu[:ff]) * gu[ff:]).to(x.dtype).to(F64)
+                if gated:
+                    act = (gu[:ff] * torch.sigmoid(gu[:ff]) * gu[ff:]).to(x.dtype).to(F64)
+                else:
+                    act = (torch.relu(gu) ** 2).to(x.dtype).to(F64)
                 out[t] += wt[t, c] * (w_down[e].to(F64) @ act)
         return out.to(torch.float32)
+
+    def embed_positions(self, token_ids, positions, table, pos_table, out):
+        out.copy_((table[token_ids.long()].to(F64) + pos_table[positions.long()].to(F64)).to(out.dtype))
+
+    def post_norm_add(self, h, y, post_weight, eps, mult, history=None, n_history=0, mix=None, next_weight=None, h_out=None):
+        def normed(x, w):
+            mu = x.mean(-1, keepdim=True)
+            return (x - mu) / torch.sqrt(((x - mu) ** 2).mean(-1, keepdim=True) + eps) * w.to(F64)
+
+        x = h.to(F64) + mult * normed(_whole(y).to(F64), post_weight)
+        if history is not None:
+            history[n_history].copy_(x.to(history.dtype))
+            x = (mix.to(F64)[: n_history + 1, None, None] * history[: n_history + 1].to(F64)).sum(0)
+        (h if h_out is None else h_out).copy_(x.to(h.dtype))
+        if next_weight is None:
+            return None
+        return normed(x, next_weight).to(next_weight.dtype)
+
+    def ff_activation(self, z, cols, mode, out, coef=None, eps=0.0, gate_col=-1):
+        full = _whole(z).to(F64)
+        v = full[:, :cols]
+        if mode == "relu2":
+            y = torch.relu(v) ** 2
+        else:
+            n = lambda u: u / torch.sqrt((u * u).mean(-1, keepdim=True) + eps)
+            c = coef.to(F64)
+            y = c[0] * n(v) + c[1] * n(v * v) + c[2] * n(v * v * v) + c[3]
+        if gate_col >= 0:
+            y = y * torch.sigmoid(full[:, gate_col : gate_col + 1])
+        out.copy_(y.to(out.dtype))
 
     def swiglu(self, gate_up, out):
         gate_up = _whole(gate_up)

@@ -91,22 +91,29 @@ def keys_and_values(h, w, p, m, eps):
     return k.view(t, m["kv_heads"], m["dim"]), v.view(t, m["kv_heads"], m["vdim"])
 
 
-def block_attention(h, w, p, m, eps, k, v):
-    """The attention mixer on the normed input h [T, W] with the keys and values it is given."""
-    t = h.shape[0]
-    nq, nkv, dk = m["heads"], m["kv_heads"], m["dim"]
-    q = rms_norm(h @ w[p + "q"].T, w[p + "q.norm"], eps).view(t, nq, dk)
-    size = m["mask"]["size"] if m.get("mask") else None
+def sloped_block_attention(q, k, v, scale, size):
+    """q [T, heads, dk], k [T, kv heads, dk], v [T, kv heads, dv] of one sequence -> [T, heads, dv]: softmax over the
+    keys that `block_visible` allows of (q . k) * scale - slope_head * (i - j)."""
+    t, nq, _ = q.shape
+    nkv = k.shape[1]
     seen = block_visible(t, size)
     distance = (torch.arange(t)[:, None] - torch.arange(t)[None, :]).to(F64)
     slopes = head_slopes(nq)
     heads = []
     for head in range(nq):
         g = head // (nq // nkv)
-        s = (q[:, head] @ k[:, g].T) * m["scale"] - slopes[head] * distance
+        s = (q[:, head] @ k[:, g].T) * scale - slopes[head] * distance
         s = s.masked_fill(~seen, -math.inf)
         heads.append(torch.softmax(s, dim=-1) @ v[:, g])
-    return torch.cat(heads, dim=-1) @ w[p + "o"].T
+    return torch.stack(heads, dim=1)
+
+
+def block_attention(h, w, p, m, eps, k, v):
+    """The attention mixer on the normed input h [T, W] with the keys and values it is given."""
+    t = h.shape[0]
+    q = rms_norm(h @ w[p + "q"].T, w[p + "q.norm"], eps).view(t, m["heads"], m["dim"])
+    size = m["mask"]["size"] if m.get("mask") else None
+    return sloped_block_attention(q, k, v, m["scale"], size).reshape(t, -1) @ w[p + "o"].T
 
 
 def forget_gates(h, w, p):
