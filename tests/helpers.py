@@ -166,9 +166,17 @@ def worst_error(rows, ref) -> tuple[float, float, tuple]:
     return worst, scale, where
 
 
-def assert_rows_match(rows, ref, tol, what=""):
+def assert_rows_match(rows, ref, tol, what="", may_exceed=0.0):
+    """Every row within tol of the reference (as a fraction of its largest magnitude); with may_exceed, that fraction
+    of the rows (at least one) may lie beyond it: a router's choice between two experts whose scores nearly tie may
+    turn under bfloat16 rounding, and the rows behind it in the request then differ too."""
     assert rows, "nothing was compared"
     worst, scale, where = worst_error(rows, ref)
+    if may_exceed and worst > tol * scale:
+        over = sum(1 for (rid, pos), row in rows.items() if float((row.double() - ref[rid][pos]).abs().max()) > tol * scale)
+        allowed = max(1, int(may_exceed * len(rows)))
+        assert over <= allowed, f"{what}: {over} of {len(rows)} rows exceed {tol:g} x {scale:.3f} (at most {allowed} may); worst {worst:.3e} at {where}"
+        return worst / scale
     assert worst <= tol * scale, f"{what}: max |diff| {worst:.3e} at {where} exceeds {tol:g} x {scale:.3f}"
     return worst / scale
 

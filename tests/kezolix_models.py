@@ -128,10 +128,10 @@ def draw_weights(cfg: dict, seed: int, sharp: float = 3.0) -> dict[str, torch.Te
             continue
         ff, n = mlp["expert"]["ff"], mlp["router"]["experts"]
         shared = mlp.get("shared")
-        common = matrix(width, ff)
+        common_up, common_down = matrix(ff, width, 2.0), matrix(width, ff)
         for e in range(n):
-            w[f"{q}e{e}.up"] = matrix(ff, width, 2.0)
-            w[f"{q}e{e}.down"] = matrix(width, ff, 0.05) if shared else common + matrix(width, ff, 0.05)
+            w[f"{q}e{e}.up"] = matrix(ff, width) if shared else common_up + matrix(ff, width, 0.03)
+            w[f"{q}e{e}.down"] = matrix(width, ff, 0.004) if shared else common_down + matrix(width, ff, 0.015)
         w[q + "router"] = matrix(n, width, 4.0)
         w[q + "correction"] = torch.where(torch.rand(n, generator=g) < 0.5, torch.zeros(n), torch.full((n,), 0.25))
         if shared:
