@@ -418,6 +418,28 @@ def nebanex_config(width, heads, kv_heads, hd, s_heads, s_dim, s_vdim, experts, 
             "logit_softcap": 50.0, "layers": [layer] * DESIGN_LAYERS}
 
 
+# `--design kezolix`: the Kezolix design (attention within blocks of positions with a penalty per head and distance,
+# one layer on an earlier layer's keys and values; a recurrence whose forget gate is bounded below; a dense
+# feed-forward with a normed polynomial and mixtures of squared-relu experts with a gated shared expert; a layer norm
+# before and behind every branch and a weighted average over all earlier layers behind every layer) beside the Nebanex
+# model of the same sizes, whose layers hold both kinds of mixer at once, and beside the Qwen2 model of the same width,
+# heads and inner width per token.  The sizes are Nebanex's; the layers: attention + experts, recurrence + experts,
+# attention on the first layer's keys + dense, recurrence + experts.
+KEZOLIX_BLOCKS = (1024, 512)
+
+
+def kezolix_config(width, heads, kv_heads, hd, s_heads, s_dim, s_vdim, experts, top, ff, shared) -> dict:
+    moe = {"kind": "moe", "router": {"experts": experts, "top": top, "scale": 2.5}, "expert": {"ff": ff}, "shared": {"ff": shared}}
+    attention = {"heads": heads, "kv_heads": kv_heads, "dim": hd, "vdim": hd, "scale": hd ** -0.5}
+    state = {"type": "hgrn2", "mixer": {"heads": s_heads, "dim": s_dim, "vdim": s_vdim}, "mlp": moe}
+    layers = [{"type": "attention", "mixer": dict(attention, mask={"size": KEZOLIX_BLOCKS[0]}), "mlp": moe}, state,
+              {"type": "attention", "mixer": dict(attention, mask={"size": KEZOLIX_BLOCKS[1]}, kv_from=0),
+               "mlp": {"kind": "dense", "ff": top * ff + shared}}, state]
+    assert len(layers) == DESIGN_LAYERS
+    return {"architecture": "Kezolix", "vocab": DESIGN_VOCAB, "width": width, "max_positions": 8192, "norm": {"eps": 1e-6},
+            "residual_mult": 0.5, "layers": layers}
+
+
 def design_models(design):
     """(label, {name: config}) for every size of the comparison, and how the sizes are named in the record."""
     if design == "pekasun":
@@ -428,9 +450,10 @@ def design_models(design):
     else:
         keys = ("width", "heads", "kv_heads", "head", "state_heads", "state_key", "state_value", "experts", "chosen",
                 "expert_inner", "shared_inner")
+        make = kezolix_config if design == "kezolix" else nebanex_config
         for s in NEBANEX_SIZES:
             label, width, heads, kv_heads, hd = s[:5]
-            yield label, dict(zip(keys, s[1:])), nebanex_config(*s[1:]), (width, s[9] * s[10] + s[11], heads, kv_heads, hd)
+            yield label, dict(zip(keys, s[1:])), make(*s[1:]), (width, s[9] * s[10] + s[11], heads, kv_heads, hd)
 
 
 def design_comparison(args) -> dict:
@@ -447,6 +470,7 @@ def design_comparison(args) -> dict:
         sizes[label] = named
         models = {
             design: design_cfg,
+            **({"nebanex": nebanex_config(*next(s for s in NEBANEX_SIZES if s[0] == label)[1:])} if design == "kezolix" else {}),
             "qwen2": dict(QWEN25_05B, hidden_size=width, intermediate_size=inner, num_attention_heads=heads,
                           num_key_value_heads=kv_heads, head_dim=hd, num_hidden_layers=DESIGN_LAYERS, vocab_size=DESIGN_VOCAB,
                           tie_word_embeddings=False),
@@ -512,9 +536,9 @@ def main() -> int:
     ap.add_argument("--no-lookahead", action="store_true",
                     help="wait for a step's tokens on the host before the next step is launched (the scheduler with --serve, "
                          "the decode loop otherwise)")
-    ap.add_argument("--design", default=None, choices=["pekasun", "nebanex"],
+    ap.add_argument("--design", default=None, choices=["pekasun", "nebanex", "kezolix"],
                     help="instead of the record: prefill and decode of that design at a few layer sizes beside the Qwen2 "
-                         "model of equal sizes")
+                         "model of equal sizes (kezolix: also beside the Nebanex model of equal sizes)")
     ap.add_argument("--direct-loop", action="store_true",
                     help="decode with the engine's step function in a loop of the benchmark's own instead of Scheduler.step")
     args = ap.parse_args()
