@@ -82,7 +82,26 @@ CONFIG_D = config(199, 96, 700, 1e-5, 0.7, [
     layer(attention(6, 3, 16, 16, 0.2, None, kv_from=0), moe(4, 2, 32, 48, 1.0)),
     layer(attention(2, 2, 48, 32, 0.15, 33), dense(64)),
 ])
-CONFIGS = {"A": (CONFIG_A, 5), "B": (CONFIG_B, 6), "C": (CONFIG_C, 7), "D": (CONFIG_D, 8)}
+# recurrences alone (no pages at all), the last one without a feed-forward
+CONFIG_F = config(150, 72, 300, 1e-5, 0.9, [
+    layer(recurrence(2, 8, 8), dense(40)),
+    layer(recurrence(1, 24, 40), moe(3, 2, 24, 8, 1.0)),
+    layer(recurrence(4, 16, 8), None),
+])
+# a deeper one: nine layers, two layers with keys of their own that are not the first ones, each read by two later
+# layers with blocks of their own (one with no blocks), three query heads per key/value head, a recurrence between
+CONFIG_G = config(321, 80, 500, 1e-5, 0.4, [
+    layer(recurrence(2, 16, 16), dense(48)),
+    layer(attention(6, 2, 16, 32, 0.2, 37), None),
+    layer(attention(6, 2, 16, 32, 0.25, 9, kv_from=1), dense(40)),
+    layer(attention(2, 2, 24, 16, 0.2, 64), moe(4, 2, 24, 16, 1.0)),
+    layer(recurrence(2, 16, 16), None),
+    layer(attention(6, 2, 16, 32, 0.3, None, kv_from=1), moe(5, 2, 16, None, 2.0)),
+    layer(attention(2, 2, 24, 16, 0.3, 16, kv_from=3), dense(40)),
+    layer(attention(2, 2, 24, 16, 0.15, 150, kv_from=3), None),
+    layer(recurrence(5, 8, 16), dense(56)),
+])
+CONFIGS = {"A": (CONFIG_A, 5), "B": (CONFIG_B, 6), "C": (CONFIG_C, 7), "D": (CONFIG_D, 8), "F": (CONFIG_F, 10), "G": (CONFIG_G, 11)}
 
 
 def draw_weights(cfg: dict, seed: int, sharp: float = 3.0) -> dict[str, torch.Tensor]:

@@ -60,7 +60,7 @@ def plain_rows(model_dir, reqs):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E", "F", "G"])
 def test_every_cutting_agrees_with_plain(models, name, dtype):
     cfg = ALL[name][0]
     reqs = H.make_requests(cfg["vocab"], [150, 1, 47, 2, 96], seed=21)

@@ -209,7 +209,7 @@ def test_the_depth_average_reads_every_earlier_result(models):
 
 
 # ----------------------------------------------------------------------------- the engine's bookkeeping
-@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "F", "G"])
 def test_cuttings_agree_with_plain(models, emulated, name):
     cfg = KM.CONFIGS[name][0]
     reqs = H.make_requests(cfg["vocab"], [5, 41, 1, 23], seed=11)
