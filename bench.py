@@ -425,7 +425,7 @@ def nebanex_config(width, heads, kv_heads, hd, s_heads, s_dim, s_vdim, experts, 
 # model of the same sizes, whose layers hold both kinds of mixer at once, and beside the Qwen2 model of the same width,
 # heads and inner width per token.  The sizes are Nebanex's; the layers: attention + experts, recurrence + experts,
 # attention on the first layer's keys + dense, recurrence + experts.
-KEZOLIX_BLOCKS = (1024, 512)
+KEZOLIX_BLOCKS = (1536, 768)       # (behind 2,048 tokens a decoded token sees 512 keys and more in both)
 
 
 def kezolix_config(width, heads, kv_heads, hd, s_heads, s_dim, s_vdim, experts, top, ff, shared) -> dict:
