@@ -1,2 +1,2 @@
 """Built-in architectures; importing this package registers them."""
-from . import kezolix, nebanex, pekasun, qwen2  # noqa: F401
+from . import bubetar, kezolix, nebanex, pekasun, qwen2  # noqa: F401

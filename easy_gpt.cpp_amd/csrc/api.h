@@ -132,19 +132,26 @@ int egpt_embed_rmsnorm(const int32_t* ids, const void* table, const void* weight
 // heads are divided by their root mean square and multiplied by q_weight / k_weight [dk] (null: the heads pass as they
 // are), value heads are divided by theirs if norm_values != 0.  Queries to q_out [n_tokens][nq * dk]; keys
 // [pages][nkv][page_size][dk] and values [pages][nkv][dv][page_size] to slots[t] (null: not stored).
+// Rows are row_width values wide.  flags: 1 the value heads are normed (the norm_values of the text above), 2 query and
+// key heads are divided by their root mean square also without weights, 4 the norm comes behind the rotation, 8 there
+// are no value columns and value head g is key head g as projected (dv == dk), 16 the rotation pairs place 2i with
+// 2i + 1 instead of i with i + rot_dims / 2.  rot_dims > 0: the first rot_dims places of query and key heads turn by
+// the angles in cos_sin float32 [n_tokens][rot_dims / 2][2] (cos, sin; both times mag).
 int egpt_head_norm_store(const void* proj, int n_splits, const float* row_ss, int ss_splits, int hidden, float norm_eps,
-                         void* q_out, const void* q_weight, const void* k_weight, float eps,
-                         int norm_values, const int32_t* slots, void* k_cache, void* v_cache, int n_tokens, int nq,
-                         int nkv, int dk, int dv, int page_size, int dtype, void* stream);
+                         int row_width, void* q_out, const void* q_weight, const void* k_weight, float eps, int flags,
+                         const float* cos_sin, int rot_dims, float mag, const int32_t* slots, void* k_cache, void* v_cache,
+                         int n_tokens, int nq, int nkv, int dk, int dv, int page_size, int dtype, void* stream);
 // proj rows of row_width values: [nq heads of (dim | rot) | rank | rot | ...].  q_plain [n_tokens][nq][dim] takes the
 // heads' unrotated parts; q_full [n_tokens][nq][rank + rot] their rotated parts behind the first rank places.  The
 // latent (normed with c_weight [rank]) and the rotated shared key are stored as key [pages][1][page_size][rank + rot],
 // the latent also as value [pages][1][rank][page_size].  cos_sin float32 [n_tokens][rot_dims / 2][2], multiplied by
 // mag; pairs (2i, 2i + 1) of the first rot_dims places of a rotated part are rotated.
+// queries (may be null): the query heads as a product of their own, rows [nq heads of (dim | rot)] (q_splits > 0: float32
+// partial sums); the latent then begins at place `lead` of proj's rows.
 int egpt_latent_prep(const void* proj, int n_splits, const float* row_ss, int ss_splits, int hidden, float norm_eps,
-                     int row_width, void* q_plain, void* q_full, const void* c_weight,
-                     float eps, const float* cos_sin, float mag, int rot_dims, const int32_t* slots, void* k_cache,
-                     void* v_cache, int n_tokens, int nq, int dim, int rot, int rank, int page_size, int dtype,
+                     int row_width, const void* queries, int q_splits, int lead, void* q_plain, void* q_full,
+                     const void* c_weight, float eps, const float* cos_sin, float mag, int rot_dims, const int32_t* slots,
+                     void* k_cache, void* v_cache, int n_tokens, int nq, int dim, int rot, int rank, int page_size, int dtype,
                      void* stream);
 // out [n_tokens][n] = x * sigmoid(gate[:, gate_off : gate_off + n]); x [n_tokens][n], or with heads > 0
 // [heads][n_tokens][n / heads]; gate: rows of gate_width values (gate_splits > 0: float32 partial sums).
@@ -184,9 +191,10 @@ int egpt_add_layernorm(float* h, const void* delta, int delta_splits, int delta_
                        void* stream);
 // out = factor * (rmsnorm(a + bias_a) * wa + rmsnorm(b + bias_b) * wb) in float32 [n_rows][hidden]; a and b are products
 // (one tensor or float32 partial sums), the biases may be null.
+// (factor weighs a, factor_b weighs b; wa and wb both null: the branches are not normed, out = factor * a + factor_b * b)
 int egpt_normed_pair_mean(const void* a, int a_splits, const void* b, int b_splits, const void* bias_a, const void* bias_b,
-                          const void* wa, const void* wb, float eps, float factor, float* out, int n_rows, int hidden,
-                          int dtype, void* stream);
+                          const void* wa, const void* wb, float eps, float factor, float factor_b, float* out, int n_rows,
+                          int hidden, int dtype, void* stream);
 // out[t] = table[ids[t]] + pos_table[positions[t]] as the float32 residual stream.
 int egpt_embed_positions(const int32_t* ids, const int32_t* positions, const void* table, const void* pos_table, float* out,
                          int n_tokens, int hidden, int vocab, int max_pos, int dtype, void* stream);
@@ -197,7 +205,8 @@ int egpt_post_norm_add(const float* h, const void* y, int y_splits, const void* 
                        int n_hist, const float* mix, float* h_out, const void* next_w, void* out, int n_rows, int hidden,
                        int dtype, void* stream);
 // x = cap * tanh(x / cap) in place.
-int egpt_tanh_cap(float* x, float cap, long long n, void* stream);
+// x <- x * scale; then, with cap > 0, x <- cap * tanh(x / cap)
+int egpt_tanh_cap(float* x, float scale, float cap, long long n, void* stream);
 // ---- head_prep.hip: norms over a whole projection, a position factor on the queries, the store into pages
 int egpt_whole_norm_store(const void* proj, int n_splits, int row_width, const void* bias, void* q_out,
                           const void* q_weight, const void* k_weight, float eps, const int32_t* positions, float coef,
@@ -205,12 +214,16 @@ int egpt_whole_norm_store(const void* proj, int n_splits, int row_width, const v
                           int dk, int dv, int page_size, int dtype, void* stream);
 // out = per-head rmsnorm(x) * weight[dv] * silu(gate columns gate_off.. of a product row); x float32 [n_tokens][heads][dv]
 // (x_splits 0) or partial sums [x_splits][n_tokens][heads][dv]; gate null: no gate
-int egpt_head_norm_gate(const float* x, int x_splits, const void* weight, float eps, const void* gate, int gate_splits, int gate_width,
-                        int gate_off, void* out, int n_tokens, int heads, int dv, int dtype, void* stream);
+// (x rows are x_width values wide, the heads from place 0; x_is_act: x is one tensor of the activation type; gate_act: 0
+// silu, 1 sigmoid, 2 the gate's columns are the factor itself)
+int egpt_head_norm_gate(const void* x, int x_splits, int x_is_act, int x_width, const void* weight, float eps, const void* gate,
+                        int gate_splits, int gate_width, int gate_off, int gate_act, void* out, int n_tokens, int heads, int dv,
+                        int dtype, void* stream);
 // ---- linear_recurrence.hip: a matrix state per head that decays per key channel
 // decay[t][c] = sigmoid(z)^(1 / tau), z = bias[c] + sum_r w[c][r] * low[t][r]; low: columns low_off.. of a product row.
+// (rates float32 [channels], may be null: the exponent per channel in place of 1 / tau; negate: z changes its sign first)
 int egpt_channel_decay(const void* low, int low_splits, int low_width, int low_off, int rank, const void* w, const void* bias,
-                       float tau, float* decay, int n_tokens, int channels, int dtype, void* stream);
+                       float tau, const float* rates, int negate, float* decay, int n_tokens, int channels, int dtype, void* stream);
 // gate[t][c] = lower[c] + (1 - lower[c]) * sigmoid(z[t][z_off + c] + bias[c]), float32 (bias, lower may be null: 0).
 int egpt_bounded_gate(const void* z, int z_splits, int z_width, int z_off, const void* bias, const void* lower, float* gate,
                       int n_tokens, int channels, int dtype, void* stream);
@@ -223,7 +236,24 @@ int egpt_scan_key_splits(int dk);
 int egpt_decayed_state_scan(const void* proj, int n_splits, int proj_width, int q_off, int k_off, int v_off, float q_scale,
                             const float* decay, float* states, const int32_t* slots, const unsigned char* fresh,
                             const int32_t* q_start, const int32_t* q_len, int n_seqs, int n_tokens, float* out, int heads,
-                            int dk, int dv, int q_silu, int tied_keys, int dtype, void* stream);
+                            int dk, int dv, int q_silu, int tied_keys, int k_silu, int v_silu, const float* head_decay,
+                            int dtype, void* stream);
+// The columns col0.. of a product row as inputs of `channels` short causal convolutions over time (weights [channels][taps],
+// the last tap the current token's; the taps - 1 inputs before a step's first token come from the request's record and
+// the record is brought up to date behind), SiLU, unit vectors head by head over the first unit_heads * unit_dim channels
+// (the first scaled_heads of them times scale), and the sigmoid of n_sig further columns: float32 [n_tokens][channels + n_sig].
+int egpt_short_conv(const void* proj, int n_splits, int proj_width, int col0, const void* conv_w, int taps, int channels,
+                    int unit_heads, int unit_dim, int scaled_heads, float scale, float unit_eps, int sig_off, int n_sig,
+                    float* states, long long state_stride, const int32_t* slots, const unsigned char* fresh,
+                    const int32_t* q_start, const int32_t* q_len, int n_seqs, int max_q_len, int n_tokens, float* out, int dtype,
+                    void* stream);
+// S <- diag(g_t) S; u = beta_t (v_t - S^T k_t); S <- S + k_t u^T; o_t = S^T q_t, token by token for every request of the step.
+// ops float32 rows hold queries and keys [kv_heads][dk], values [heads][dv] and beta [heads] at their offsets; decay float32
+// [n_tokens][heads * dk]; value head h reads query/key head h / (heads / kv_heads); out float32 [n_tokens][heads * dv].
+int egpt_delta_rule_scan(const float* ops, int ops_width, int q_off, int k_off, int v_off, int beta_off, const float* decay,
+                         float* states, long long state_stride, const int32_t* slots, const unsigned char* fresh,
+                         const int32_t* q_start, const int32_t* q_len, int n_seqs, int n_tokens, float* out, int heads,
+                         int kv_heads, int dk, int dv, void* stream);
 // ---- moe.hip: a mixture of gated experts
 // logits = x router^T + bias in float32; the `top` largest per token (lowest index among equals) to chosen[t][top], the
 // softmax over the chosen logits to weight[t][top].

@@ -49,34 +49,66 @@ __global__ __launch_bounds__(256) void embed_rmsnorm_kernel(const int32_t* __res
     for (int j = threadIdx.x; j < hidden; j += blockDim.x) residual_store(o + j, to_float(row[j]) * inv * to_float(weight[j]));
 }
 
-// One wavefront per (token, head) of a product row [nq heads of dk | nkv heads of dk | nkv heads of dv]: a query or
-// key head is divided by its root mean square and multiplied by the weight that all heads share (a null weight:
-// the head passes as it is), a value head is divided by its root mean square if norm_values is set.  Queries go
-// to q_out [T][nq * dk]; keys and values to the pages at slots[t] (slots null: nothing is stored).
+// One wavefront per (token, head) of a product row [nq heads of dk | nkv heads of dk | nkv heads of dv | anything else]
+// of row_width values: a query or key head is divided by its root mean square and multiplied by the weight that all
+// heads share (a null weight: the head passes as it is, or with kNormPlain it is divided and no more), a value head
+// is divided by its root mean square if kNormValues is set.  With kValuesAreKeys the row holds no value heads: value
+// head g is key head g as it was projected (dv == dk).  Queries and keys are rotated when rot_dims > 0: the first
+// rot_dims places of a head turn by the angles whose (cos, sin) stand in cos_sin [T][rot_dims / 2][2] (both times mag),
+// place i with place i + rot_dims / 2, or with kInterleaved place 2i with place 2i + 1; behind the norm, or with
+// kNormAfterRotation before it.  Queries go to q_out [T][nq * dk]; keys and values to the pages at slots[t] (slots
+// null: nothing is stored).
+constexpr int kNormValues = 1, kNormPlain = 2, kNormAfterRotation = 4, kValuesAreKeys = 8, kInterleaved = 16;
+
 template <typename T>
 __global__ __launch_bounds__(kWave) void head_norm_store_kernel(
-    ProductView<T> proj, RowFactor factor, T* __restrict__ q_out, const T* __restrict__ q_weight,
-    const T* __restrict__ k_weight, float eps, int norm_values, const int32_t* __restrict__ slots, T* __restrict__ k_cache, T* __restrict__ v_cache, int nq, int nkv,
+    ProductView<T> proj, RowFactor factor, int row_width, T* __restrict__ q_out, const T* __restrict__ q_weight,
+    const T* __restrict__ k_weight, float eps, int flags, const float* __restrict__ cos_sin, int rot_dims, float mag,
+    const int32_t* __restrict__ slots, T* __restrict__ k_cache, T* __restrict__ v_cache, int nq, int nkv,
     int dk, int dv, int page_size) {
     const int t = blockIdx.x, hh = blockIdx.y, lane = threadIdx.x;
-    const int row_width = (nq + nkv) * dk + nkv * dv;
     const int kind = hh < nq ? 0 : (hh < nq + nkv ? 1 : 2);
     const int head = kind == 0 ? hh : (kind == 1 ? hh - nq : hh - nq - nkv);
     const int width = kind == 2 ? dv : dk;
-    const int in_off = kind == 0 ? head * dk : (kind == 1 ? nq * dk + head * dk : (nq + nkv) * dk + head * dv);
+    const bool own_keys = kind == 2 && (flags & kValuesAreKeys);
+    const int in_off = kind == 0 ? head * dk : ((kind == 1 || own_keys) ? nq * dk + head * dk : (nq + nkv) * dk + head * dv);
     if (kind != 0 && slots == nullptr) return;
     const T* weight = kind == 0 ? q_weight : (kind == 1 ? k_weight : nullptr);
-    const bool normed = kind == 2 ? norm_values != 0 : weight != nullptr;
+    const bool normed = kind == 2 ? (flags & kNormValues) != 0 : (weight != nullptr || (flags & kNormPlain));
+    const int rot = kind == 2 ? 0 : rot_dims;
+    const int half = rot / 2;
+    const bool interleaved = (flags & kInterleaved) != 0;
+    const bool norm_after = (flags & kNormAfterRotation) != 0;
     const size_t base = static_cast<size_t>(t) * row_width + in_off;
+    const float* cs = cos_sin + static_cast<size_t>(t) * rot_dims;
     const float rf = factor.of(t);
-    float v[kOwn];
+    float v[kOwn], pv[kOwn];
     float ss = 0.f;
 #pragma unroll
     for (int r = 0; r < kOwn; ++r) {
         const int d = lane + r * kWave;
         v[r] = d < width ? proj.at(base + d) * rf : 0.f;
-        ss = fmaf(v[r], v[r], ss);
+        pv[r] = 0.f;
+        if (d < rot) {                                    // the place this one turns with
+            const int pd = interleaved ? (d ^ 1) : (d < half ? d + half : d - half);
+            pv[r] = proj.at(base + pd) * rf;
+        }
     }
+    auto turn = [&](int d, float own, float other) {
+        const int i = interleaved ? d / 2 : (d < half ? d : d - half);
+        const bool first = interleaved ? (d & 1) == 0 : d < half;
+        const float c = cs[2 * i] * mag, s = cs[2 * i + 1] * mag;
+        return first ? __fmaf_rn(own, c, -__fmul_rn(other, s)) : __fmaf_rn(other, s, __fmul_rn(own, c));
+    };
+    if (norm_after) {
+#pragma unroll
+        for (int r = 0; r < kOwn; ++r) {
+            const int d = lane + r * kWave;
+            if (d < rot) v[r] = turn(d, v[r], pv[r]);
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < kOwn; ++r) ss = fmaf(v[r], v[r], ss);
     float inv = 1.0f;
     if (normed) inv = inv_rms(wave_sum(ss), 1.0f / static_cast<float>(width), eps);
     long page = 0;
@@ -91,6 +123,12 @@ __global__ __launch_bounds__(kWave) void head_norm_store_kernel(
         if (d >= width) continue;
         float y = v[r] * inv;
         if (weight != nullptr) y *= to_float(weight[d]);
+        if (d < rot && !norm_after) {
+            const int pd = interleaved ? (d ^ 1) : (d < half ? d + half : d - half);
+            float py = pv[r] * inv;
+            if (weight != nullptr) py *= to_float(weight[pd]);
+            y = turn(d, y, py);
+        }
         if (kind == 0)
             q_out[static_cast<size_t>(t) * nq * dk + head * dk + d] = from_float<T>(y);
         else if (kind == 1)
@@ -102,6 +140,8 @@ __global__ __launch_bounds__(kWave) void head_norm_store_kernel(
 
 // One wavefront per (token, query head) and one more per token for the latent, of a product row
 // [nq heads of (dim unrotated | rot rotated) | rank latent | rot shared rotated key | anything else].
+// With qsrc present the query heads are the rows [nq heads of (dim | rot)] of that product instead, and the latent begins
+// at place `lead` of proj's row (behind whatever stands there in the queries' stead).
 // A query head's unrotated part goes to q_plain [T][nq][dim], its rotated part, rotated, to q_full [T][nq][rank + rot]
 // behind the first rank places (which the caller fills with the unrotated part carried into the latent space).
 // The latent is divided by its root mean square and multiplied by c_weight; with the rotated shared key behind it
@@ -110,7 +150,7 @@ __global__ __launch_bounds__(kWave) void head_norm_store_kernel(
 // cos_sin [T][rot_dims / 2][2]; both are multiplied by mag; places from rot_dims on pass unchanged.
 template <typename T>
 __global__ __launch_bounds__(kWave) void latent_prep_kernel(
-    ProductView<T> proj, RowFactor factor, int row_width, T* __restrict__ q_plain, T* __restrict__ q_full,
+    ProductView<T> proj, RowFactor factor, int row_width, ProductView<T> qsrc, int lead, T* __restrict__ q_plain, T* __restrict__ q_full,
     const T* __restrict__ c_weight, float eps, const float* __restrict__ cos_sin, float mag, int rot_dims, const int32_t* __restrict__ slots,
     T* __restrict__ k_cache, T* __restrict__ v_cache, int nq, int dim, int rot, int rank, int page_size) {
     const int t = blockIdx.x, hh = blockIdx.y, lane = threadIdx.x;
@@ -119,22 +159,25 @@ __global__ __launch_bounds__(kWave) void latent_prep_kernel(
     const int dk = rank + rot;
     const float rf = factor.of(t);
     if (hh < nq) {
-        const size_t base = row + static_cast<size_t>(hh) * (dim + rot);
+        const bool own = qsrc.present();
+        const ProductView<T>& src = own ? qsrc : proj;
+        const float qf = own ? 1.0f : rf;
+        const size_t base = (own ? static_cast<size_t>(t) * nq * (dim + rot) : row) + static_cast<size_t>(hh) * (dim + rot);
         for (int d = lane; d < dim; d += kWave)
-            q_plain[(static_cast<size_t>(t) * nq + hh) * dim + d] = from_float<T>(proj.at(base + d) * rf);
+            q_plain[(static_cast<size_t>(t) * nq + hh) * dim + d] = from_float<T>(src.at(base + d) * qf);
         T* dst = q_full + (static_cast<size_t>(t) * nq + hh) * dk + rank;
         for (int i = lane; i < rot / 2; i += kWave) {
-            const float u = proj.at(base + dim + 2 * i) * rf, w = proj.at(base + dim + 2 * i + 1) * rf;
+            const float u = src.at(base + dim + 2 * i) * qf, w = src.at(base + dim + 2 * i + 1) * qf;
             float ru = u, rw = w;
             if (2 * i + 1 < rot_dims) rotate_pair(u, w, cs[2 * i] * mag, cs[2 * i + 1] * mag, ru, rw);
             dst[2 * i] = from_float<T>(ru);
             dst[2 * i + 1] = from_float<T>(rw);
         }
-        if ((rot & 1) && lane == 0) dst[rot - 1] = from_float<T>(proj.at(base + dim + rot - 1) * rf);
+        if ((rot & 1) && lane == 0) dst[rot - 1] = from_float<T>(src.at(base + dim + rot - 1) * qf);
         return;
     }
     if (slots == nullptr) return;
-    const size_t base = row + static_cast<size_t>(nq) * (dim + rot);
+    const size_t base = row + static_cast<size_t>(lead);
     float v[kOwn];
     float ss = 0.f;
 #pragma unroll
@@ -270,26 +313,31 @@ __global__ __launch_bounds__(256) void whole_norm_store_kernel(
     }
 }
 
-// out[t][h * dv + d] = x[t][h * dv + d] / rms(x[t][h * dv ..]) * weight[d] * silu(g[t][gate_off + h * dv + d]): the
-// RMS norm of every head's float32 output (one tensor, or partial sums that are added here) with a weight that the heads share, and a SiLU gate from columns of a
-// product row (no gate: the normed heads as they are).  One wavefront per (token, head).
+// out[t][h * dv + d] = x[t][h * dv + d] / rms(x[t][h * dv ..]) * weight[d] * act(g[t][gate_off + h * dv + d]): the
+// RMS norm of every head's output with a weight that the heads share, and a gate from columns of a product row (no
+// gate: the normed heads as they are).  x is float32 (one tensor, or partial sums that are added here) or, with xa
+// present, a product in the activation type; its rows are x_width values wide and the heads begin at place 0.  The
+// gate's activation: 0 silu, 1 sigmoid, 2 none (the columns hold the factor itself).  One wavefront per (token, head).
 template <typename T>
-__global__ __launch_bounds__(kWave) void head_norm_gate_kernel(ProductView<float> x, const T* __restrict__ weight,
-                                                               float eps, ProductView<T> g, int gate_width, int gate_off,
-                                                               T* __restrict__ out, int heads, int dv) {
+__global__ __launch_bounds__(kWave) void head_norm_gate_kernel(ProductView<float> x, ProductView<T> xa, int x_width,
+                                                               const T* __restrict__ weight, float eps, ProductView<T> g,
+                                                               int gate_width, int gate_off, int gate_act, T* __restrict__ out,
+                                                               int heads, int dv) {
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-    const size_t xr = (static_cast<size_t>(t) * heads + h) * dv;
+    const size_t xr = static_cast<size_t>(t) * x_width + static_cast<size_t>(h) * dv;
+    const bool act_typed = xa.present();
     float ss = 0.f;
     for (int d = lane; d < dv; d += kWave) {
-        const float v = x.at(xr + d);
+        const float v = act_typed ? xa.at(xr + d) : x.at(xr + d);
         ss = fmaf(v, v, ss);
     }
     const float inv = inv_rms(wave_sum(ss), 1.0f / static_cast<float>(dv), eps);
     for (int d = lane; d < dv; d += kWave) {
-        float y = x.at(xr + d) * inv * to_float(weight[d]);
+        float y = (act_typed ? xa.at(xr + d) : x.at(xr + d)) * inv * to_float(weight[d]);
         if (g.present()) {
             const float gate = g.at(static_cast<size_t>(t) * gate_width + gate_off + h * dv + d);
-            y *= gate / (1.0f + expf(-gate));
+            const float sig = 1.0f / (1.0f + expf(-gate));
+            y *= gate_act == 0 ? gate * sig : (gate_act == 1 ? sig : gate);
         }
         out[(static_cast<size_t>(t) * heads + h) * dv + d] = from_float<T>(y);
     }
@@ -332,38 +380,41 @@ extern "C" int egpt_embed_rmsnorm(const int32_t* ids, const void* table, const v
 }
 
 extern "C" int egpt_head_norm_store(const void* proj, int n_splits, const float* row_ss, int ss_splits, int hidden,
-                                    float norm_eps, void* q_out, const void* q_weight,
-                                    const void* k_weight, float eps, int norm_values, const int32_t* slots,
-                                    void* k_cache, void* v_cache, int n_tokens, int nq, int nkv, int dk, int dv,
-                                    int page_size, int dtype, void* stream) {
+                                    float norm_eps, int row_width, void* q_out, const void* q_weight,
+                                    const void* k_weight, float eps, int flags, const float* cos_sin, int rot_dims, float mag,
+                                    const int32_t* slots, void* k_cache, void* v_cache, int n_tokens, int nq, int nkv, int dk,
+                                    int dv, int page_size, int dtype, void* stream) {
     if (!proj || !q_out || n_splits < 0 || n_tokens < 0 || nq <= 0 || nkv <= 0 || dk <= 0 || dv <= 0 || page_size <= 0 ||
-        (dtype != 0 && dtype != 1))
+        (dtype != 0 && dtype != 1) || flags < 0 || flags >= 32)
         return EGPT_BAD_ARGUMENT;
     if (slots && (!k_cache || !v_cache)) return EGPT_BAD_ARGUMENT;
+    if (rot_dims < 0 || rot_dims % 2 || rot_dims > dk || (rot_dims > 0 && !cos_sin)) return EGPT_BAD_ARGUMENT;
+    if ((flags & kValuesAreKeys) && (dv != dk || (flags & kNormValues))) return EGPT_BAD_ARGUMENT;
+    if (row_width < (nq + nkv) * dk + ((flags & kValuesAreKeys) ? 0 : nkv * dv)) return EGPT_BAD_ARGUMENT;
     if (dk > kMaxHeadWidth || dv > kMaxHeadWidth || nq + 2 * nkv > 65535) return EGPT_UNSUPPORTED_SIZE;
     if (n_tokens == 0) return EGPT_OK;
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (row_ss && (n_splits < 1 || ss_splits < 1 || hidden <= 0)) return EGPT_BAD_ARGUMENT;
     const RowFactor factor{row_ss, ss_splits, n_tokens, hidden, norm_eps};
-    const size_t stride = static_cast<size_t>(n_tokens) * ((nq + nkv) * dk + nkv * dv);
+    const size_t stride = static_cast<size_t>(n_tokens) * row_width;
     dim3 grid(n_tokens, nq + 2 * nkv);
     if (dtype == 0)
         head_norm_store_kernel<float><<<grid, kWave, 0, s>>>(
-            view_of<float>(proj, n_splits, stride), factor, static_cast<float*>(q_out), static_cast<const float*>(q_weight),
-            static_cast<const float*>(k_weight), eps, norm_values, slots, static_cast<float*>(k_cache),
+            view_of<float>(proj, n_splits, stride), factor, row_width, static_cast<float*>(q_out), static_cast<const float*>(q_weight),
+            static_cast<const float*>(k_weight), eps, flags, cos_sin, rot_dims, mag, slots, static_cast<float*>(k_cache),
             static_cast<float*>(v_cache), nq, nkv, dk, dv, page_size);
     else
         head_norm_store_kernel<bf16_t><<<grid, kWave, 0, s>>>(
-            view_of<bf16_t>(proj, n_splits, stride), factor, static_cast<bf16_t*>(q_out), static_cast<const bf16_t*>(q_weight),
-            static_cast<const bf16_t*>(k_weight), eps, norm_values, slots, static_cast<bf16_t*>(k_cache),
+            view_of<bf16_t>(proj, n_splits, stride), factor, row_width, static_cast<bf16_t*>(q_out), static_cast<const bf16_t*>(q_weight),
+            static_cast<const bf16_t*>(k_weight), eps, flags, cos_sin, rot_dims, mag, slots, static_cast<bf16_t*>(k_cache),
             static_cast<bf16_t*>(v_cache), nq, nkv, dk, dv, page_size);
     EGPT_CHECK_LAUNCH();
     return EGPT_OK;
 }
 
 extern "C" int egpt_latent_prep(const void* proj, int n_splits, const float* row_ss, int ss_splits, int hidden,
-                                float norm_eps, int row_width, void* q_plain, void* q_full,
-                                const void* c_weight, float eps, const float* cos_sin, float mag, int rot_dims,
+                                float norm_eps, int row_width, const void* queries, int q_splits, int lead, void* q_plain,
+                                void* q_full, const void* c_weight, float eps, const float* cos_sin, float mag, int rot_dims,
                                 const int32_t* slots, void* k_cache, void* v_cache, int n_tokens, int nq, int dim,
                                 int rot, int rank, int page_size, int dtype, void* stream) {
     if (!proj || !q_plain || !q_full || !c_weight || n_splits < 0 || n_tokens < 0 || nq <= 0 || dim <= 0 || rot < 0 ||
@@ -371,23 +422,26 @@ extern "C" int egpt_latent_prep(const void* proj, int n_splits, const float* row
         return EGPT_BAD_ARGUMENT;
     if (rot_dims > 0 && !cos_sin) return EGPT_BAD_ARGUMENT;
     if (slots && (!k_cache || !v_cache)) return EGPT_BAD_ARGUMENT;
-    if (row_width < nq * (dim + rot) + rank + rot) return EGPT_BAD_ARGUMENT;
+    if (!queries) lead = nq * (dim + rot);
+    if (lead < 0 || q_splits < 0 || row_width < lead + rank + rot) return EGPT_BAD_ARGUMENT;
     if (rank > kMaxHeadWidth || nq + 1 > 65535) return EGPT_UNSUPPORTED_SIZE;
     if (n_tokens == 0) return EGPT_OK;
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (row_ss && (n_splits < 1 || ss_splits < 1 || hidden <= 0)) return EGPT_BAD_ARGUMENT;
     const RowFactor factor{row_ss, ss_splits, n_tokens, hidden, norm_eps};
     const size_t stride = static_cast<size_t>(n_tokens) * row_width;
+    const size_t q_stride = static_cast<size_t>(n_tokens) * nq * (dim + rot);
     dim3 grid(n_tokens, nq + 1);
     if (dtype == 0)
         latent_prep_kernel<float><<<grid, kWave, 0, s>>>(
-            view_of<float>(proj, n_splits, stride), factor, row_width, static_cast<float*>(q_plain), static_cast<float*>(q_full),
+            view_of<float>(proj, n_splits, stride), factor, row_width, view_of<float>(queries, queries ? q_splits : 0, q_stride), lead,
+            static_cast<float*>(q_plain), static_cast<float*>(q_full),
             static_cast<const float*>(c_weight), eps, cos_sin, mag, rot_dims, slots, static_cast<float*>(k_cache),
             static_cast<float*>(v_cache), nq, dim, rot, rank, page_size);
     else
         latent_prep_kernel<bf16_t><<<grid, kWave, 0, s>>>(
-            view_of<bf16_t>(proj, n_splits, stride), factor, row_width, static_cast<bf16_t*>(q_plain),
-            static_cast<bf16_t*>(q_full), static_cast<const bf16_t*>(c_weight), eps, cos_sin, mag, rot_dims, slots,
+            view_of<bf16_t>(proj, n_splits, stride), factor, row_width, view_of<bf16_t>(queries, queries ? q_splits : 0, q_stride), lead,
+            static_cast<bf16_t*>(q_plain), static_cast<bf16_t*>(q_full), static_cast<const bf16_t*>(c_weight), eps, cos_sin, mag, rot_dims, slots,
             static_cast<bf16_t*>(k_cache), static_cast<bf16_t*>(v_cache), nq, dim, rot, rank, page_size);
     EGPT_CHECK_LAUNCH();
     return EGPT_OK;
@@ -446,10 +500,11 @@ extern "C" int egpt_whole_norm_store(const void* proj, int n_splits, int row_wid
     return EGPT_OK;
 }
 
-extern "C" int egpt_head_norm_gate(const float* x, int x_splits, const void* weight, float eps, const void* gate, int gate_splits,
-                                   int gate_width, int gate_off, void* out, int n_tokens, int heads, int dv, int dtype,
-                                   void* stream) {
-    if (!x || x_splits < 0 || !weight || !out || n_tokens < 0 || heads <= 0 || dv <= 0 || gate_splits < 0 || (dtype != 0 && dtype != 1))
+extern "C" int egpt_head_norm_gate(const void* x, int x_splits, int x_is_act, int x_width, const void* weight, float eps,
+                                   const void* gate, int gate_splits, int gate_width, int gate_off, int gate_act, void* out,
+                                   int n_tokens, int heads, int dv, int dtype, void* stream) {
+    if (!x || x_splits < 0 || !weight || !out || n_tokens < 0 || heads <= 0 || dv <= 0 || gate_splits < 0 || (dtype != 0 && dtype != 1) ||
+        gate_act < 0 || gate_act > 2 || x_width < heads * dv || (x_is_act && x_splits != 0))
         return EGPT_BAD_ARGUMENT;
     if (gate && (gate_off < 0 || gate_off + heads * dv > gate_width)) return EGPT_BAD_ARGUMENT;
     if (!gate) gate_splits = 0;
@@ -458,19 +513,21 @@ extern "C" int egpt_head_norm_gate(const float* x, int x_splits, const void* wei
     hipStream_t s = static_cast<hipStream_t>(stream);
     const size_t stride = static_cast<size_t>(n_tokens) * gate_width;
     dim3 grid(n_tokens, heads);
-    // x float32 [n_tokens][heads * dv] (x_splits 0) or partial sums [x_splits][n_tokens][heads * dv]
+    // x float32 [n_tokens][x_width] (x_splits 0) or partial sums [x_splits][n_tokens][x_width]; or of the activation type
     ProductView<float> xv;
-    xv.whole = x_splits == 0 ? x : nullptr;
-    xv.partial = x_splits > 0 ? x : nullptr;
+    xv.whole = (x_splits == 0 && !x_is_act) ? static_cast<const float*>(x) : nullptr;
+    xv.partial = x_splits > 0 ? static_cast<const float*>(x) : nullptr;
     xv.n_splits = x_splits;
-    xv.split_stride = static_cast<size_t>(n_tokens) * heads * dv;
+    xv.split_stride = static_cast<size_t>(n_tokens) * x_width;
     if (dtype == 0)
-        head_norm_gate_kernel<float><<<grid, kWave, 0, s>>>(xv, static_cast<const float*>(weight), eps,
-                                                            view_of<float>(gate, gate_splits, stride), gate_width, gate_off,
+        head_norm_gate_kernel<float><<<grid, kWave, 0, s>>>(xv, view_of<float>(x_is_act ? x : nullptr, 0, 0), x_width,
+                                                            static_cast<const float*>(weight), eps,
+                                                            view_of<float>(gate, gate_splits, stride), gate_width, gate_off, gate_act,
                                                             static_cast<float*>(out), heads, dv);
     else
-        head_norm_gate_kernel<bf16_t><<<grid, kWave, 0, s>>>(xv, static_cast<const bf16_t*>(weight), eps,
-                                                             view_of<bf16_t>(gate, gate_splits, stride), gate_width, gate_off,
+        head_norm_gate_kernel<bf16_t><<<grid, kWave, 0, s>>>(xv, view_of<bf16_t>(x_is_act ? x : nullptr, 0, 0), x_width,
+                                                             static_cast<const bf16_t*>(weight), eps,
+                                                             view_of<bf16_t>(gate, gate_splits, stride), gate_width, gate_off, gate_act,
                                                              static_cast<bf16_t*>(out), heads, dv);
     EGPT_CHECK_LAUNCH();
     return EGPT_OK;

@@ -6,8 +6,14 @@
 //
 // egpt_channel_decay makes the decays a = sigmoid(z)^(1/tau) from a low-rank projection (z = W low + b);
 // egpt_bounded_gate makes decays with a learned lower bound, a = l + (1 - l) sigmoid(z + b), from columns of a product;
-// egpt_decayed_state_scan runs the recurrence; its queries may pass through SiLU on their way in, and its keys may be
-// tied to the decays, k = 1 - a (a forget gate that also sets what is written), instead of columns of the product.
+// egpt_decayed_state_scan runs the recurrence; its queries, keys and values may each pass through SiLU on their way in,
+// its keys may be tied to the decays, k = 1 - a (a forget gate that also sets what is written), instead of columns of
+// the product, and its decay may be one constant per head.
+//
+// The delta rule, S <- diag(g_t) S; u_t = beta_t (v_t - S^T k_t); S <- S + k_t u_t^T; o_t = S^T q_t, mixes the key channels in
+// every token (S^T k), so its scan keeps a head's whole key range in one workgroup: egpt_delta_rule_scan.  Its operands
+// come from egpt_short_conv, which runs the short causal convolutions over time with their carried inputs, SiLU, and the
+// unit norms of queries and keys.
 #include "api.h"
 #include "common.h"
 
@@ -28,10 +34,13 @@ ProductView<T> scan_view(const void* p, int n_splits, size_t stride) {
 constexpr int kMaxRank = 1024;
 
 // One workgroup per token: the token's low-rank vector in LDS, a thread per channel.
-// sigmoid(z)^(1/tau) = exp(-softplus(-z) / tau), with softplus(-z) = max(-z, 0) + log1p(exp(-|z|)).
+// sigmoid(z)^(1/tau) = exp(-softplus(-z) / tau), with softplus(-z) = max(-z, 0) + log1p(exp(-|z|)).  With rates the
+// exponent is rates[c] per channel instead of 1/tau, and with negate z changes its sign first, which together give
+// exp(-rate softplus(z)) = sigmoid(-z)^rate: a decay whose logarithm is a step size times a rate per channel.
 template <typename T>
 __global__ __launch_bounds__(256) void channel_decay_kernel(ProductView<T> low, int low_width, int low_off, int rank,
                                                             const T* __restrict__ w, const T* __restrict__ bias, float inv_tau,
+                                                            const float* __restrict__ rates, int negate,
                                                             float* __restrict__ decay, int channels) {
     __shared__ float low_s[kMaxRank];
     const int t = blockIdx.x;
@@ -41,8 +50,9 @@ __global__ __launch_bounds__(256) void channel_decay_kernel(ProductView<T> low, 
         float z = bias ? to_float(bias[c]) : 0.f;
         const T* wr = w + static_cast<size_t>(c) * rank;
         for (int r = 0; r < rank; ++r) z = fmaf(to_float(wr[r]), low_s[r], z);
+        if (negate) z = -z;
         const float log_sigmoid = -(fmaxf(-z, 0.f) + log1pf(expf(-fabsf(z))));
-        decay[static_cast<size_t>(t) * channels + c] = expf(log_sigmoid * inv_tau);
+        decay[static_cast<size_t>(t) * channels + c] = expf(log_sigmoid * (rates ? rates[c] : inv_tau));
     }
 }
 
@@ -79,7 +89,7 @@ __global__ __launch_bounds__(64 * kScanWaves) void decayed_state_scan_kernel(
     ProductView<T> proj, int proj_width, int q_off, int k_off, int v_off, float q_scale, const float* __restrict__ decay,
     float* __restrict__ states, const int32_t* __restrict__ slots, const unsigned char* __restrict__ fresh,
     const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len, float* __restrict__ out, int n_tokens, int heads,
-    int dk, int dv, int key_splits, int q_silu, int tied_keys) {
+    int dk, int dv, int key_splits, int q_silu, int tied_keys, int k_silu, int v_silu, const float* __restrict__ head_decay) {
     constexpr int NS = kScanWaves, DKR = kScanKeys / kScanWaves, THREADS = 64 * NS, DKP = kScanKeys;
     constexpr int QKA = kScanTokens * DKP / THREADS;          // values of q (or k, or decays) of a batch per thread
     constexpr int VL = kScanTokens * kScanCols / THREADS;     // values of v, and outputs, of a batch per thread
@@ -118,7 +128,7 @@ __global__ __launch_bounds__(64 * kScanWaves) void decayed_state_scan_kernel(
             if (tt < count && r < dk) {
                 const size_t row = static_cast<size_t>(t0 + base + tt);
                 rq[u] = proj.at(row * proj_width + q_off + h * dk + r);      // (scaled when it is staged: nothing here waits for a load)
-                ra[u] = decay[row * channels + h * dk + r];
+                ra[u] = head_decay ? head_decay[h] : decay[row * channels + h * dk + r];
                 if (!tied_keys) rk[u] = proj.at(row * proj_width + k_off + h * dk + r);
             }
         }
@@ -140,11 +150,11 @@ __global__ __launch_bounds__(64 * kScanWaves) void decayed_state_scan_kernel(
             // (a tied key is 1 - a; a place that holds no token or no channel has a = 0 and would get k = 1, which meets a
             // query of zero and a state row that is never stored)
             q_s[tid + u * THREADS] = (q_silu ? rq[u] / (1.0f + expf(-rq[u])) : rq[u]) * q_scale;
-            k_s[tid + u * THREADS] = tied_keys ? 1.0f - ra[u] : rk[u];
+            k_s[tid + u * THREADS] = tied_keys ? 1.0f - ra[u] : (k_silu ? rk[u] / (1.0f + expf(-rk[u])) : rk[u]);
             a_s[tid + u * THREADS] = ra[u];
         }
 #pragma unroll
-        for (int u = 0; u < VL; ++u) v_s[tid + u * THREADS] = rv[u];
+        for (int u = 0; u < VL; ++u) v_s[tid + u * THREADS] = v_silu ? rv[u] / (1.0f + expf(-rv[u])) : rv[u];
         __syncthreads();
         if (base + kScanTokens < n) fetch(base + kScanTokens);
         for (int tt = 0; tt < count; ++tt) {
@@ -185,7 +195,8 @@ __global__ __launch_bounds__(64 * kScanWaves) void decayed_state_scan_kernel(
 using namespace egpt;
 
 extern "C" int egpt_channel_decay(const void* low, int low_splits, int low_width, int low_off, int rank, const void* w,
-                                  const void* bias, float tau, float* decay, int n_tokens, int channels, int dtype, void* stream) {
+                                  const void* bias, float tau, const float* rates, int negate, float* decay, int n_tokens,
+                                  int channels, int dtype, void* stream) {
     if (!low || !w || !decay || low_splits < 0 || rank <= 0 || low_off < 0 || low_off + rank > low_width || n_tokens < 0 ||
         channels <= 0 || !(tau > 0.f) || (dtype != 0 && dtype != 1))
         return EGPT_BAD_ARGUMENT;
@@ -196,11 +207,11 @@ extern "C" int egpt_channel_decay(const void* low, int low_splits, int low_width
     if (dtype == 0)
         channel_decay_kernel<float><<<n_tokens, 256, 0, s>>>(scan_view<float>(low, low_splits, stride), low_width, low_off, rank,
                                                              static_cast<const float*>(w), static_cast<const float*>(bias),
-                                                             1.0f / tau, decay, channels);
+                                                             1.0f / tau, rates, negate, decay, channels);
     else
         channel_decay_kernel<bf16_t><<<n_tokens, 256, 0, s>>>(scan_view<bf16_t>(low, low_splits, stride), low_width, low_off, rank,
                                                               static_cast<const bf16_t*>(w), static_cast<const bf16_t*>(bias),
-                                                              1.0f / tau, decay, channels);
+                                                              1.0f / tau, rates, negate, decay, channels);
     EGPT_CHECK_LAUNCH();
     return EGPT_OK;
 }
@@ -230,13 +241,13 @@ template <typename T>
 static int launch_scan(const void* proj, int n_splits, int proj_width, int q_off, int k_off, int v_off, float q_scale,
                        const float* decay, float* states, const int32_t* slots, const unsigned char* fresh,
                        const int32_t* q_start, const int32_t* q_len, int n_seqs, int n_tokens, float* out, int heads, int dk,
-                       int dv, int q_silu, int tied_keys, hipStream_t s) {
+                       int dv, int q_silu, int tied_keys, int k_silu, int v_silu, const float* head_decay, hipStream_t s) {
     const ProductView<T> view = scan_view<T>(proj, n_splits, static_cast<size_t>(n_tokens) * proj_width);
     const int key_splits = (dk + kScanKeys - 1) / kScanKeys;
     dim3 grid(n_seqs, heads, (dv + kScanCols - 1) / kScanCols * key_splits);
     decayed_state_scan_kernel<T><<<grid, 64 * kScanWaves, 0, s>>>(view, proj_width, q_off, k_off, v_off, q_scale, decay, states, slots,
                                                                   fresh, q_start, q_len, out, n_tokens, heads, dk, dv, key_splits,
-                                                                  q_silu, tied_keys);
+                                                                  q_silu, tied_keys, k_silu, v_silu, head_decay);
     return EGPT_OK;
 }
 
@@ -246,8 +257,9 @@ extern "C" int egpt_decayed_state_scan(const void* proj, int n_splits, int proj_
                                        float q_scale, const float* decay, float* states, const int32_t* slots,
                                        const unsigned char* fresh, const int32_t* q_start, const int32_t* q_len, int n_seqs,
                                        int n_tokens, float* out, int heads, int dk, int dv, int q_silu, int tied_keys,
-                                       int dtype, void* stream) {
-    if (!proj || !decay || !states || !slots || !q_start || !q_len || !out || n_splits < 0 || n_seqs <= 0 || n_tokens < 0 ||
+                                       int k_silu, int v_silu, const float* head_decay, int dtype, void* stream) {
+    // head_decay float32 [heads]: one constant decay per head in place of the decays per token and key channel
+    if (!proj || (!decay && !head_decay) || (tied_keys && k_silu) || !states || !slots || !q_start || !q_len || !out || n_splits < 0 || n_seqs <= 0 || n_tokens < 0 ||
         heads <= 0 || dk <= 0 || dv <= 0 || q_off < 0 || (!tied_keys && k_off < 0) || v_off < 0 || (dtype != 0 && dtype != 1))
         return EGPT_BAD_ARGUMENT;
     if (q_off + heads * dk > proj_width || (!tied_keys && k_off + heads * dk > proj_width) || v_off + heads * dv > proj_width)
@@ -258,10 +270,293 @@ extern "C" int egpt_decayed_state_scan(const void* proj, int n_splits, int proj_
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype == 0)
         launch_scan<float>(proj, n_splits, proj_width, q_off, k_off, v_off, q_scale, decay, states, slots, fresh, q_start,
-                           q_len, n_seqs, n_tokens, out, heads, dk, dv, q_silu, tied_keys, s);
+                           q_len, n_seqs, n_tokens, out, heads, dk, dv, q_silu, tied_keys, k_silu, v_silu, head_decay, s);
     else
         launch_scan<bf16_t>(proj, n_splits, proj_width, q_off, k_off, v_off, q_scale, decay, states, slots, fresh, q_start,
-                            q_len, n_seqs, n_tokens, out, heads, dk, dv, q_silu, tied_keys, s);
+                            q_len, n_seqs, n_tokens, out, heads, dk, dv, q_silu, tied_keys, k_silu, v_silu, head_decay, s);
+    EGPT_CHECK_LAUNCH();
+    return EGPT_OK;
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
+// Short causal convolutions over time, and the delta rule's scan.
+namespace egpt {
+
+constexpr int kMaxTaps = 16;
+
+// One workgroup per token of a step (grid: requests x the step's longest portion).  The columns col0 .. col0 + channels
+// of a product row are the inputs of `channels` independent convolutions over time: y_i = sum_j w[c][j] x_(i - taps + 1 + j)
+// (the last tap is the current token's), with the inputs before the step's first token taken from the request's record
+// hist [taps - 1][channels] (zeros for a request that starts anew).  y passes SiLU.  The first unit_heads * unit_dim
+// channels are then made unit vectors head by head, y / sqrt(sum y^2 + unit_eps), the first scaled_heads of them also
+// times `scale`.  Behind the channels the output row holds the sigmoid of the n_sig columns from sig_off on.  All float32.
+template <typename T>
+__global__ __launch_bounds__(256) void short_conv_kernel(
+    ProductView<T> proj, int proj_width, int col0, const T* __restrict__ conv_w, int taps, int channels, int unit_heads,
+    int unit_dim, int scaled_heads, float scale, float unit_eps, int sig_off, int n_sig, const float* __restrict__ states,
+    size_t state_stride, const int32_t* __restrict__ slots, const unsigned char* __restrict__ fresh,
+    const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len, float* __restrict__ out, int out_width) {
+    extern __shared__ float conv_s[];
+    const int b = blockIdx.x, i = blockIdx.y;
+    if (i >= q_len[b]) return;
+    const int t0 = q_start[b];
+    const size_t t = static_cast<size_t>(t0 + i);
+    const float* hist = states + static_cast<size_t>(slots[b]) * state_stride;
+    const bool anew = fresh != nullptr && fresh[b] != 0;
+    for (int c = threadIdx.x; c < channels; c += blockDim.x) {
+        float acc = 0.f;
+        for (int j = 0; j < taps; ++j) {
+            const int src = i - (taps - 1) + j;
+            float x;
+            if (src >= 0)
+                x = proj.at(static_cast<size_t>(t0 + src) * proj_width + col0 + c);
+            else
+                x = anew ? 0.f : hist[static_cast<size_t>(src + taps - 1) * channels + c];
+            acc = fmaf(x, to_float(conv_w[static_cast<size_t>(c) * taps + j]), acc);
+        }
+        conv_s[c] = acc / (1.0f + expf(-acc));
+    }
+    __syncthreads();
+    float* orow = out + t * out_width;
+    const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave, n_waves = blockDim.x / kWave;
+    for (int hh = wave; hh < unit_heads; hh += n_waves) {
+        const float* head = conv_s + hh * unit_dim;
+        float ss = 0.f;
+        for (int d = lane; d < unit_dim; d += kWave) ss = fmaf(head[d], head[d], ss);
+        float f = 1.0f / sqrtf(wave_sum(ss) + unit_eps);
+        if (hh < scaled_heads) f *= scale;
+        for (int d = lane; d < unit_dim; d += kWave) orow[hh * unit_dim + d] = head[d] * f;
+    }
+    for (int c = unit_heads * unit_dim + threadIdx.x; c < channels; c += blockDim.x) orow[c] = conv_s[c];
+    for (int c = threadIdx.x; c < n_sig; c += blockDim.x)
+        orow[channels + c] = 1.0f / (1.0f + expf(-proj.at(t * proj_width + sig_off + c)));
+}
+
+// After a step: a request's record takes the last taps - 1 inputs of its convolutions (those of this step, and, where the
+// step brought fewer, what the record held, moved up).  One workgroup per request; a thread owns a channel's column.
+template <typename T>
+__global__ __launch_bounds__(256) void conv_carry_kernel(ProductView<T> proj, int proj_width, int col0, int taps, int channels,
+                                                         float* __restrict__ states, size_t state_stride,
+                                                         const int32_t* __restrict__ slots, const unsigned char* __restrict__ fresh,
+                                                         const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len) {
+    const int b = blockIdx.x;
+    const int n = q_len[b];
+    if (n <= 0) return;
+    const int t0 = q_start[b];
+    float* hist = states + static_cast<size_t>(slots[b]) * state_stride;
+    const bool anew = fresh != nullptr && fresh[b] != 0;
+    for (int c = threadIdx.x; c < channels; c += blockDim.x) {
+        float keep[kMaxTaps];
+#pragma unroll
+        for (int j = 0; j < kMaxTaps; ++j) {
+            keep[j] = 0.f;
+            if (j < taps - 1) {
+                const int src = n - (taps - 1) + j;
+                if (src >= 0)
+                    keep[j] = proj.at(static_cast<size_t>(t0 + src) * proj_width + col0 + c);
+                else if (!anew)
+                    keep[j] = hist[static_cast<size_t>(src + taps - 1) * channels + c];
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < kMaxTaps; ++j)
+            if (j < taps - 1) hist[static_cast<size_t>(j) * channels + c] = keep[j];
+    }
+}
+
+// One workgroup per (request, head, 64 value channels); a lane is a column of the head's state S [dk][dv], and wavefront w
+// keeps the key channels w * DKR .. of that column in registers.  Per token: the column decays row by row, every wavefront
+// sums its rows' part of S^T k, the parts meet in LDS (two buffers in turn, so one barrier a token), u = beta (v - S^T k),
+// the rows take k u, and the wavefronts' parts of S^T q are kept for the end of the batch, where they are added in the
+// order of the wavefronts.  A batch of `tb` tokens' operands is staged in LDS.  Value head h reads the queries and keys of
+// head h / (heads / kv_heads).  ops rows hold queries, keys, values and beta (float32); decay is [tokens][heads * dk].
+template <int DKR>
+__global__ __launch_bounds__(1024) void delta_rule_scan_kernel(
+    const float* __restrict__ ops, int ops_width, int q_off, int k_off, int v_off, int beta_off, const float* __restrict__ decay,
+    float* __restrict__ states, size_t state_stride, const int32_t* __restrict__ slots, const unsigned char* __restrict__ fresh,
+    const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len, float* __restrict__ out, int heads, int kv_heads,
+    int dk, int dv, int tb) {
+    extern __shared__ __attribute__((aligned(16))) float scan_s[];
+    const int nw = blockDim.x / kWave, dkp = nw * DKR;
+    float* q_s = scan_s;
+    float* k_s = q_s + tb * dkp;
+    float* g_s = k_s + tb * dkp;
+    float* v_s = g_s + tb * dkp;
+    float* beta_s = v_s + tb * kScanCols;
+    float* part_s = beta_s + ((tb + 3) & ~3);
+    float* red_s = part_s + tb * nw * kScanCols;
+    const int b = blockIdx.x, h = blockIdx.y, col0 = blockIdx.z * kScanCols;
+    const int n = q_len[b];
+    if (n <= 0) return;
+    const int t0 = q_start[b];
+    const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+    const int j = col0 + lane;
+    const bool has_col = j < dv;
+    const int kvh = h / (heads / kv_heads);
+    float* state = states + static_cast<size_t>(slots[b]) * state_stride + static_cast<size_t>(h) * dk * dv;
+    const bool anew = fresh != nullptr && fresh[b] != 0;
+    float s[DKR];
+#pragma unroll
+    for (int i = 0; i < DKR; ++i) {
+        const int r = wave * DKR + i;
+        s[i] = (!anew && has_col && r < dk) ? state[static_cast<size_t>(r) * dv + j] : 0.f;
+    }
+    const int threads = blockDim.x;
+    for (int base = 0; base < n; base += tb) {
+        const int count = min(tb, n - base);
+        __syncthreads();                              // the batch before is read, its parts are added
+        for (int idx = tid; idx < count * dkp; idx += threads) {
+            const int tt = idx / dkp, r = idx % dkp;
+            const size_t row = static_cast<size_t>(t0 + base + tt);
+            const bool valid = r < dk;
+            q_s[idx] = valid ? ops[row * ops_width + q_off + kvh * dk + r] : 0.f;
+            k_s[idx] = valid ? ops[row * ops_width + k_off + kvh * dk + r] : 0.f;
+            g_s[idx] = valid ? decay[row * heads * dk + static_cast<size_t>(h) * dk + r] : 0.f;
+        }
+        for (int idx = tid; idx < count * kScanCols; idx += threads) {
+            const int tt = idx / kScanCols, c = idx % kScanCols;
+            const size_t row = static_cast<size_t>(t0 + base + tt);
+            v_s[idx] = col0 + c < dv ? ops[row * ops_width + v_off + h * dv + col0 + c] : 0.f;
+        }
+        for (int idx = tid; idx < count; idx += threads)
+            beta_s[idx] = ops[static_cast<size_t>(t0 + base + idx) * ops_width + beta_off + h];
+        __syncthreads();
+        for (int tt = 0; tt < count; ++tt) {
+            const float4* g4 = reinterpret_cast<const float4*>(g_s + tt * dkp + wave * DKR);
+            const float4* k4 = reinterpret_cast<const float4*>(k_s + tt * dkp + wave * DKR);
+            const float4* q4 = reinterpret_cast<const float4*>(q_s + tt * dkp + wave * DKR);
+            float kk[DKR];
+            float p = 0.f;
+#pragma unroll
+            for (int i = 0; i < DKR / 4; ++i) {
+                const float4 g = g4[i], k = k4[i];
+                kk[4 * i] = k.x, kk[4 * i + 1] = k.y, kk[4 * i + 2] = k.z, kk[4 * i + 3] = k.w;
+                s[4 * i] *= g.x, s[4 * i + 1] *= g.y, s[4 * i + 2] *= g.z, s[4 * i + 3] *= g.w;
+                p = fmaf(s[4 * i], k.x, p);
+                p = fmaf(s[4 * i + 1], k.y, p);
+                p = fmaf(s[4 * i + 2], k.z, p);
+                p = fmaf(s[4 * i + 3], k.w, p);
+            }
+            float* red = red_s + (tt & 1) * nw * kScanCols;
+            red[wave * kScanCols + lane] = p;
+            __syncthreads();
+            float total = 0.f;
+            for (int w = 0; w < nw; ++w) total += red[w * kScanCols + lane];
+            const float u = beta_s[tt] * (v_s[tt * kScanCols + lane] - total);
+            float po = 0.f;
+#pragma unroll
+            for (int i = 0; i < DKR / 4; ++i) {
+                const float4 q = q4[i];
+                s[4 * i] = fmaf(kk[4 * i], u, s[4 * i]);
+                s[4 * i + 1] = fmaf(kk[4 * i + 1], u, s[4 * i + 1]);
+                s[4 * i + 2] = fmaf(kk[4 * i + 2], u, s[4 * i + 2]);
+                s[4 * i + 3] = fmaf(kk[4 * i + 3], u, s[4 * i + 3]);
+                po = fmaf(s[4 * i], q.x, po);
+                po = fmaf(s[4 * i + 1], q.y, po);
+                po = fmaf(s[4 * i + 2], q.z, po);
+                po = fmaf(s[4 * i + 3], q.w, po);
+            }
+            part_s[(tt * nw + wave) * kScanCols + lane] = po;
+        }
+        __syncthreads();
+        for (int idx = tid; idx < count * kScanCols; idx += threads) {
+            const int tt = idx / kScanCols, c = idx % kScanCols;
+            if (col0 + c < dv) {
+                float o = 0.f;
+                for (int w = 0; w < nw; ++w) o += part_s[(tt * nw + w) * kScanCols + c];
+                out[(static_cast<size_t>(t0 + base + tt) * heads + h) * dv + col0 + c] = o;
+            }
+        }
+    }
+    if (has_col) {
+#pragma unroll
+        for (int i = 0; i < DKR; ++i) {
+            const int r = wave * DKR + i;
+            if (r < dk) state[static_cast<size_t>(r) * dv + j] = s[i];
+        }
+    }
+}
+
+}  // namespace egpt
+
+// out float32 [n_tokens][channels + n_sig]; states: the first record's convolution inputs [taps - 1][channels], a
+// request's record lies state_stride floats further per slot.  The records are brought up to date behind the step's
+// convolutions (a second launch on the same stream).
+extern "C" int egpt_short_conv(const void* proj, int n_splits, int proj_width, int col0, const void* conv_w, int taps,
+                               int channels, int unit_heads, int unit_dim, int scaled_heads, float scale, float unit_eps,
+                               int sig_off, int n_sig, float* states, long long state_stride, const int32_t* slots,
+                               const unsigned char* fresh, const int32_t* q_start, const int32_t* q_len, int n_seqs,
+                               int max_q_len, int n_tokens, float* out, int dtype, void* stream) {
+    if (!proj || !conv_w || !states || !slots || !q_start || !q_len || !out || n_splits < 0 || taps < 1 || channels <= 0 ||
+        unit_heads < 0 || unit_dim < 0 || scaled_heads < 0 || scaled_heads > unit_heads || n_sig < 0 || col0 < 0 || n_seqs <= 0 ||
+        max_q_len < 0 || n_tokens < 0 || (dtype != 0 && dtype != 1))
+        return EGPT_BAD_ARGUMENT;
+    if (static_cast<long long>(unit_heads) * unit_dim > channels || col0 + channels > proj_width ||
+        (n_sig > 0 && (sig_off < 0 || sig_off + n_sig > proj_width)) || state_stride < static_cast<long long>(taps - 1) * channels)
+        return EGPT_BAD_ARGUMENT;
+    if (taps > kMaxTaps || channels > 15360 || max_q_len > 65535) return EGPT_UNSUPPORTED_SIZE;     // a token's channels lie in LDS
+    if (n_tokens == 0 || max_q_len == 0) return EGPT_OK;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const size_t stride = static_cast<size_t>(n_tokens) * proj_width;
+    const size_t lds = static_cast<size_t>(channels) * sizeof(float);
+    const int out_width = channels + n_sig;
+    dim3 grid(n_seqs, max_q_len);
+    if (dtype == 0) {
+        short_conv_kernel<float><<<grid, 256, lds, s>>>(scan_view<float>(proj, n_splits, stride), proj_width, col0,
+                                                        static_cast<const float*>(conv_w), taps, channels, unit_heads, unit_dim,
+                                                        scaled_heads, scale, unit_eps, sig_off, n_sig, states,
+                                                        static_cast<size_t>(state_stride), slots, fresh, q_start, q_len, out, out_width);
+        if (taps > 1)
+            conv_carry_kernel<float><<<n_seqs, 256, 0, s>>>(scan_view<float>(proj, n_splits, stride), proj_width, col0, taps, channels,
+                                                            states, static_cast<size_t>(state_stride), slots, fresh, q_start, q_len);
+    } else {
+        short_conv_kernel<bf16_t><<<grid, 256, lds, s>>>(scan_view<bf16_t>(proj, n_splits, stride), proj_width, col0,
+                                                         static_cast<const bf16_t*>(conv_w), taps, channels, unit_heads, unit_dim,
+                                                         scaled_heads, scale, unit_eps, sig_off, n_sig, states,
+                                                         static_cast<size_t>(state_stride), slots, fresh, q_start, q_len, out, out_width);
+        if (taps > 1)
+            conv_carry_kernel<bf16_t><<<n_seqs, 256, 0, s>>>(scan_view<bf16_t>(proj, n_splits, stride), proj_width, col0, taps, channels,
+                                                             states, static_cast<size_t>(state_stride), slots, fresh, q_start, q_len);
+    }
+    EGPT_CHECK_LAUNCH();
+    return EGPT_OK;
+}
+
+// out float32 [n_tokens][heads * dv]; states: the first record's matrices [heads][dk][dv], a request's record lies
+// state_stride floats further per slot.
+extern "C" int egpt_delta_rule_scan(const float* ops, int ops_width, int q_off, int k_off, int v_off, int beta_off,
+                                    const float* decay, float* states, long long state_stride, const int32_t* slots,
+                                    const unsigned char* fresh, const int32_t* q_start, const int32_t* q_len, int n_seqs,
+                                    int n_tokens, float* out, int heads, int kv_heads, int dk, int dv, void* stream) {
+    if (!ops || !decay || !states || !slots || !q_start || !q_len || !out || n_seqs <= 0 || n_tokens < 0 || heads <= 0 ||
+        kv_heads <= 0 || heads % kv_heads || dk <= 0 || dv <= 0 || q_off < 0 || k_off < 0 || v_off < 0 || beta_off < 0)
+        return EGPT_BAD_ARGUMENT;
+    if (q_off + kv_heads * dk > ops_width || k_off + kv_heads * dk > ops_width || v_off + heads * dv > ops_width ||
+        beta_off + heads > ops_width || state_stride < static_cast<long long>(heads) * dk * dv)
+        return EGPT_BAD_ARGUMENT;
+    if (dk > 1024 || heads > 65535 || (dv + kScanCols - 1) / kScanCols > 65535) return EGPT_UNSUPPORTED_SIZE;
+    if (n_tokens == 0) return EGPT_OK;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    // rows of the state per wavefront, and wavefronts per workgroup (at most 16)
+    const int dkr = dk <= 256 ? 16 : (dk <= 512 ? 32 : 64);
+    const int nw = (dk + dkr - 1) / dkr, dkp = nw * dkr;
+    // as many tokens to a batch as fit 60 KB of LDS beside the two buffers in which the wavefronts' sums meet
+    const size_t per_token = (3 * static_cast<size_t>(dkp) + kScanCols + static_cast<size_t>(nw) * kScanCols) * sizeof(float) + 4;
+    const size_t fixed = (2 * static_cast<size_t>(nw) * kScanCols + 4) * sizeof(float);
+    int tb = static_cast<int>((60 * 1024 - fixed) / per_token);
+    tb = tb > 32 ? 32 : (tb < 1 ? 1 : tb);
+    const size_t lds = fixed + per_token * tb + 16;
+    dim3 grid(n_seqs, heads, (dv + kScanCols - 1) / kScanCols);
+    const size_t stride = static_cast<size_t>(state_stride);
+    if (dkr == 16)
+        delta_rule_scan_kernel<16><<<grid, nw * kWave, lds, s>>>(ops, ops_width, q_off, k_off, v_off, beta_off, decay, states, stride,
+                                                                 slots, fresh, q_start, q_len, out, heads, kv_heads, dk, dv, tb);
+    else if (dkr == 32)
+        delta_rule_scan_kernel<32><<<grid, nw * kWave, lds, s>>>(ops, ops_width, q_off, k_off, v_off, beta_off, decay, states, stride,
+                                                                 slots, fresh, q_start, q_len, out, heads, kv_heads, dk, dv, tb);
+    else
+        delta_rule_scan_kernel<64><<<grid, nw * kWave, lds, s>>>(ops, ops_width, q_off, k_off, v_off, beta_off, decay, states, stride,
+                                                                 slots, fresh, q_start, q_len, out, heads, kv_heads, dk, dv, tb);
     EGPT_CHECK_LAUNCH();
     return EGPT_OK;
 }

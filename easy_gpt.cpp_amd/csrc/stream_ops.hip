@@ -69,12 +69,13 @@ __global__ __launch_bounds__(256) void add_layernorm_kernel(float* __restrict__ 
     }
 }
 
-// out[t, :] = factor * (a[t, :] / rms(a[t, :]) * wa + b[t, :] / rms(b[t, :]) * wb), float32: what two branches
-// that are normed before they are joined leave for the residual stream.
+// out[t, :] = factor_a * a[t, :] / rms(a[t, :]) * wa + factor_b * b[t, :] / rms(b[t, :]) * wb, float32: what two branches
+// that are normed before they are joined leave for the residual stream.  Without weights (wa null) the branches are not
+// normed: out = factor_a * a + factor_b * b.
 template <typename T>
 __global__ __launch_bounds__(256) void normed_pair_mean_kernel(ProductView<T> a, ProductView<T> b, const T* __restrict__ bias_a,
                                                                const T* __restrict__ bias_b, const T* __restrict__ wa,
-                                                               const T* __restrict__ wb, float eps, float factor,
+                                                               const T* __restrict__ wb, float eps, float factor_a, float factor_b,
                                                                float* __restrict__ out, int hidden) {
     extern __shared__ float pair_s[];
     __shared__ float scratch[16];
@@ -91,10 +92,15 @@ __global__ __launch_bounds__(256) void normed_pair_mean_kernel(ProductView<T> a,
         ssa = fmaf(x, x, ssa);
         ssb = fmaf(y, y, ssb);
     }
+    if (wa == nullptr) {
+        for (int j = threadIdx.x; j < hidden; j += blockDim.x) out[base + j] = factor_a * a_s[j] + factor_b * b_s[j];
+        return;
+    }
     const float inv_a = inv_rms(block_sum(ssa, scratch), 1.0f / static_cast<float>(hidden), eps);
     const float inv_b = inv_rms(block_sum(ssb, scratch), 1.0f / static_cast<float>(hidden), eps);
     for (int j = threadIdx.x; j < hidden; j += blockDim.x)
-        out[base + j] = factor * (a_s[j] * inv_a * to_float(wa[j]) + b_s[j] * inv_b * to_float(wb[j]));
+        out[base + j] = factor_a == factor_b ? factor_a * (a_s[j] * inv_a * to_float(wa[j]) + b_s[j] * inv_b * to_float(wb[j]))
+                                             : factor_a * (a_s[j] * inv_a * to_float(wa[j])) + factor_b * (b_s[j] * inv_b * to_float(wb[j]));
 }
 
 // x[t, :] = E[id_t, :] + P[position_t, :]: a token's vector plus a learned vector of its position, added in float32
@@ -166,10 +172,13 @@ __global__ __launch_bounds__(256) void post_norm_add_kernel(const float* h, Prod
         out[base + j] = from_float<T>((row_s[j] - mean) * inv * to_float(next_w[j]));
 }
 
-__global__ __launch_bounds__(256) void tanh_cap_kernel(float* __restrict__ x, float cap, size_t n) {
-    const float inv = 1.0f / cap;
-    for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += static_cast<size_t>(gridDim.x) * blockDim.x)
-        x[i] = cap * tanhf(x[i] * inv);
+// x <- x * scale, then (cap > 0) x <- cap * tanh(x / cap)
+__global__ __launch_bounds__(256) void tanh_cap_kernel(float* __restrict__ x, float scale, float cap, size_t n) {
+    const float inv = cap > 0.f ? 1.0f / cap : 0.f;
+    for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += static_cast<size_t>(gridDim.x) * blockDim.x) {
+        const float v = x[i] * scale;
+        x[i] = cap > 0.f ? cap * tanhf(v * inv) : v;
+    }
 }
 
 }  // namespace egpt
@@ -212,9 +221,9 @@ extern "C" int egpt_add_layernorm(float* h, const void* delta, int delta_splits,
 }
 
 extern "C" int egpt_normed_pair_mean(const void* a, int a_splits, const void* b, int b_splits, const void* bias_a,
-                                     const void* bias_b, const void* wa, const void* wb, float eps, float factor, float* out,
-                                     int n_rows, int hidden, int dtype, void* stream) {
-    if (!a || !b || !wa || !wb || !out || n_rows < 0 || hidden <= 0 || a_splits < 0 || b_splits < 0 || (dtype != 0 && dtype != 1))
+                                     const void* bias_b, const void* wa, const void* wb, float eps, float factor, float factor_b,
+                                     float* out, int n_rows, int hidden, int dtype, void* stream) {
+    if (!a || !b || (wa == nullptr) != (wb == nullptr) || !out || n_rows < 0 || hidden <= 0 || a_splits < 0 || b_splits < 0 || (dtype != 0 && dtype != 1))
         return EGPT_BAD_ARGUMENT;
     if (hidden > 8192) return EGPT_UNSUPPORTED_SIZE;           // two rows lie in LDS
     if (n_rows == 0) return EGPT_OK;
@@ -224,11 +233,11 @@ extern "C" int egpt_normed_pair_mean(const void* a, int a_splits, const void* b,
     if (dtype == 0)
         normed_pair_mean_kernel<float><<<n_rows, 256, lds, s>>>(
             stream_view<float>(a, a_splits, stride), stream_view<float>(b, b_splits, stride), static_cast<const float*>(bias_a),
-            static_cast<const float*>(bias_b), static_cast<const float*>(wa), static_cast<const float*>(wb), eps, factor, out, hidden);
+            static_cast<const float*>(bias_b), static_cast<const float*>(wa), static_cast<const float*>(wb), eps, factor, factor_b, out, hidden);
     else
         normed_pair_mean_kernel<bf16_t><<<n_rows, 256, lds, s>>>(
             stream_view<bf16_t>(a, a_splits, stride), stream_view<bf16_t>(b, b_splits, stride), static_cast<const bf16_t*>(bias_a),
-            static_cast<const bf16_t*>(bias_b), static_cast<const bf16_t*>(wa), static_cast<const bf16_t*>(wb), eps, factor, out, hidden);
+            static_cast<const bf16_t*>(bias_b), static_cast<const bf16_t*>(wa), static_cast<const bf16_t*>(wb), eps, factor, factor_b, out, hidden);
     EGPT_CHECK_LAUNCH();
     return EGPT_OK;
 }
@@ -273,12 +282,12 @@ extern "C" int egpt_post_norm_add(const float* h, const void* y, int y_splits, c
     return EGPT_OK;
 }
 
-extern "C" int egpt_tanh_cap(float* x, float cap, long long n, void* stream) {
-    if (!x || n < 0 || !(cap > 0.f)) return EGPT_BAD_ARGUMENT;
+extern "C" int egpt_tanh_cap(float* x, float scale, float cap, long long n, void* stream) {
+    if (!x || n < 0 || !(cap >= 0.f)) return EGPT_BAD_ARGUMENT;           // cap 0: the factor alone
     if (n == 0) return EGPT_OK;
     const long long blocks = (n + 255) / 256;
     tanh_cap_kernel<<<static_cast<unsigned>(blocks > 4096 ? 4096 : blocks), 256, 0, static_cast<hipStream_t>(stream)>>>(
-        x, cap, static_cast<size_t>(n));
+        x, scale, cap, static_cast<size_t>(n));
     EGPT_CHECK_LAUNCH();
     return EGPT_OK;
 }

@@ -28,7 +28,7 @@ def _load_library() -> ctypes.CDLL:
         lib = ctypes.CDLL(path)
     except (build.BuildError, OSError) as e:
         raise KernelsUnavailable(f"the HIP kernel library could not be built or loaded: {e}") from e
-    if lib.egpt_abi_version() != 22:
+    if lib.egpt_abi_version() != 23:
         raise KernelsUnavailable(f"{path} has an unexpected ABI version")
     return lib
 
@@ -102,8 +102,8 @@ class HipKernels(KernelBackend):
             "egpt_sample_wide": [vp, vp, vp, vp, vp, vp, vp, i, i, vp],
             "egpt_gemm_gate_up_swiglu": [vp, vp, vp, i, i, i, i, vp],
             "egpt_embed_rmsnorm": [vp, vp, vp, f, vp, i, i, i, i, i, vp],
-            "egpt_head_norm_store": [vp, i, vp, i, i, f, vp, vp, vp, f, i, vp, vp, vp, i, i, i, i, i, i, i, vp],
-            "egpt_latent_prep": [vp, i, vp, i, i, f, i, vp, vp, vp, f, vp, f, i, vp, vp, vp, i, i, i, i, i, i, i, vp],
+            "egpt_head_norm_store": [vp, i, vp, i, i, f, i, vp, vp, vp, f, i, vp, i, f, vp, vp, vp, i, i, i, i, i, i, i, vp],
+            "egpt_latent_prep": [vp, i, vp, i, i, f, i, vp, i, i, vp, vp, vp, f, vp, f, i, vp, vp, vp, i, i, i, i, i, i, i, vp],
             "egpt_sigmoid_gate": [vp, i, vp, i, vp, i, i, f, i, i, vp, i, i, i, vp],
             "egpt_window_attention": [vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, i, f, i, i, vp, vp, i, i, vp, i, vp],
             "egpt_window_attention_tiled": [vp, vp, vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, i, f, i, i, vp, vp, i,
@@ -115,12 +115,14 @@ class HipKernels(KernelBackend):
             "egpt_moe_up": [vp, vp, vp, vp, vp, i, i, i, i, i, i, vp],
             "egpt_embed_scaled": [vp, vp, f, vp, i, i, i, i, vp],
             "egpt_add_layernorm": [vp, vp, i, i, vp, vp, vp, f, vp, i, i, i, vp],
-            "egpt_normed_pair_mean": [vp, i, vp, i, vp, vp, vp, vp, f, f, vp, i, i, i, vp],
-            "egpt_tanh_cap": [vp, f, ctypes.c_longlong, vp],
+            "egpt_normed_pair_mean": [vp, i, vp, i, vp, vp, vp, vp, f, f, f, vp, i, i, i, vp],
+            "egpt_tanh_cap": [vp, f, f, ctypes.c_longlong, vp],
             "egpt_whole_norm_store": [vp, i, i, vp, vp, vp, vp, f, vp, f, i, vp, vp, vp, i, i, i, i, i, i, i, vp],
-            "egpt_head_norm_gate": [vp, i, vp, f, vp, i, i, i, vp, i, i, i, i, vp],
-            "egpt_channel_decay": [vp, i, i, i, i, vp, vp, f, vp, i, i, i, vp],
-            "egpt_decayed_state_scan": [vp, i, i, i, i, i, f, vp, vp, vp, vp, vp, vp, i, i, vp, i, i, i, i, i, i, vp],
+            "egpt_head_norm_gate": [vp, i, i, i, vp, f, vp, i, i, i, i, vp, i, i, i, i, vp],
+            "egpt_channel_decay": [vp, i, i, i, i, vp, vp, f, vp, i, vp, i, i, i, vp],
+            "egpt_decayed_state_scan": [vp, i, i, i, i, i, f, vp, vp, vp, vp, vp, vp, i, i, vp, i, i, i, i, i, i, i, vp, i, vp],
+            "egpt_short_conv": [vp, i, i, i, vp, i, i, i, i, i, f, f, i, i, vp, ctypes.c_longlong, vp, vp, vp, vp, i, i, i, vp, i, vp],
+            "egpt_delta_rule_scan": [vp, i, i, i, i, i, vp, vp, ctypes.c_longlong, vp, vp, vp, vp, i, i, vp, i, i, i, i, vp],
             "egpt_moe_route": [vp, vp, vp, vp, vp, i, i, i, i, i, vp, f, i, vp],
             "egpt_moe_group": [vp, vp, vp, vp, vp, i, i, i, i, vp],
             "egpt_moe_gate_up": [vp, vp, vp, vp, vp, i, i, i, i, i, i, vp],
@@ -904,31 +906,56 @@ class HipKernels(KernelBackend):
             raise ValueError("k_cache and v_cache must have the same number of pages")
 
     def head_norm_store(self, proj, q_out, q_weight, k_weight, eps, norm_values, slots, k_cache, v_cache, nq, nkv, dk, dv,
-                        page_size, row_ss=None, hidden=0, norm_eps=0.0):
+                        page_size, row_ss=None, hidden=0, norm_eps=0.0, row_width=None, cos_sin=None, rotary_dim=0,
+                        pairing="half", magnitude=1.0, norm_plain=False, norm_after_rotation=False, values_are_keys=False):
+        """row_width: the width of proj's rows when more stands behind the heads; cos_sin float32 [T, rotary_dim / 2, 2]
+        with rotary_dim > 0: query and key heads are rotated over their first rotary_dim places (pairing 'half': place i
+        with i + rotary_dim / 2; 'interleaved': 2i with 2i + 1), behind the norm or, with norm_after_rotation, before
+        it; norm_plain: the heads are divided by their root mean square without a weight; values_are_keys: no value
+        columns, a value head is its key head as projected."""
         t = proj.shape[-2]
         dt = self._act(q_out, "q_out")
-        splits = self._product(proj, "proj", q_out.dtype, t, (nq + nkv) * dk + nkv * dv)
+        used = (nq + nkv) * dk + (0 if values_are_keys else nkv * dv)
+        width = used if row_width is None else int(row_width)
+        if width < used:
+            raise ValueError(f"proj rows of {width} values cannot hold {nq} + {nkv} heads of {dk}"
+                             + ("" if values_are_keys else f" and {nkv} of {dv}"))
+        if values_are_keys and (dv != dk or norm_values):
+            raise ValueError("values that are the keys as projected have the keys' size and are not normed")
+        if pairing not in ("half", "interleaved"):
+            raise ValueError(f"unknown pairing '{pairing}' of the rotation (half, interleaved)")
+        splits = self._product(proj, "proj", q_out.dtype, t, width)
         self._need(q_out, "q_out", None, (t, nq * dk))
         for name, w in (("q_weight", q_weight), ("k_weight", k_weight)):
             if w is not None:
                 self._need(w, name, q_out.dtype, (dk,))
+        if rotary_dim:
+            if rotary_dim % 2 or not 0 < rotary_dim <= dk:
+                raise ValueError(f"rotary_dim {rotary_dim} must be even and at most the key size {dk}")
+            self._need(cos_sin, "cos_sin", _F32, (t, rotary_dim // 2, 2))
         if slots is not None:
             self._need(slots, "slots", _I32, (t,))
             self._key_value_pages(k_cache, v_cache, q_out.dtype, nkv, page_size, dk, dv)
+        flags = ((1 if norm_values else 0) | (2 if norm_plain else 0) | (4 if norm_after_rotation else 0)
+                 | (8 if values_are_keys else 0) | (16 if pairing == "interleaved" else 0))
         self._run("egpt_head_norm_store", proj.data_ptr(), splits, *self._row_factor(row_ss, splits, t, hidden, norm_eps),
-                  q_out.data_ptr(), self._ptr(q_weight),
-                  self._ptr(k_weight), float(eps), 1 if norm_values else 0, self._ptr(slots),
+                  width, q_out.data_ptr(), self._ptr(q_weight), self._ptr(k_weight), float(eps), flags,
+                  self._ptr(cos_sin) if rotary_dim else None, int(rotary_dim), float(magnitude), self._ptr(slots),
                   self._ptr(k_cache) if slots is not None else None, self._ptr(v_cache) if slots is not None else None,
                   t, nq, nkv, dk, dv, page_size, dt, self._stream())
 
     def latent_prep(self, proj, q_plain, q_full, c_weight, eps, cos_sin, magnitude, rotary_dim, slots, k_cache, v_cache,
-                    nq, dim, rot, rank, page_size, row_ss=None, hidden=0, norm_eps=0.0):
+                    nq, dim, rot, rank, page_size, row_ss=None, hidden=0, norm_eps=0.0, queries=None, lead_width=None):
+        """queries: the query heads as a product of their own, rows [nq heads of (dim | rot)]; the latent then begins at
+        place lead_width of proj's rows."""
         t, width = proj.shape[-2], proj.shape[-1]
         dt = self._act(q_full, "q_full")
-        if width < nq * (dim + rot) + rank + rot:
-            raise ValueError(f"proj rows of {width} values cannot hold {nq} heads of {dim} + {rot}, a latent of {rank} and "
+        lead = nq * (dim + rot) if queries is None else int(lead_width)
+        if lead < 0 or width < lead + rank + rot:
+            raise ValueError(f"proj rows of {width} values cannot hold {lead} leading values, a latent of {rank} and "
                              f"a rotated key of {rot}")
         splits = self._product(proj, "proj", q_full.dtype, t, width)
+        q_splits = 0 if queries is None else self._product(queries, "queries", q_full.dtype, t, nq * (dim + rot))
         self._need(q_plain, "q_plain", q_full.dtype, (t, nq, dim))
         self._need(q_full, "q_full", None, (t, nq, rank + rot))
         self._need(c_weight, "c_weight", q_full.dtype, (rank,))
@@ -940,7 +967,7 @@ class HipKernels(KernelBackend):
             self._need(slots, "slots", _I32, (t,))
             self._key_value_pages(k_cache, v_cache, q_full.dtype, 1, page_size, rank + rot, rank)
         self._run("egpt_latent_prep", proj.data_ptr(), splits, *self._row_factor(row_ss, splits, t, hidden, norm_eps),
-                  int(width), q_plain.data_ptr(), q_full.data_ptr(),
+                  int(width), self._ptr(queries), q_splits, lead, q_plain.data_ptr(), q_full.data_ptr(),
                   c_weight.data_ptr(), float(eps), self._ptr(cos_sin) if rotary_dim else None, float(magnitude),
                   int(rotary_dim), self._ptr(slots), self._ptr(k_cache) if slots is not None else None,
                   self._ptr(v_cache) if slots is not None else None, t, nq, dim, rot, rank, page_size, dt, self._stream())
@@ -1043,20 +1070,26 @@ class HipKernels(KernelBackend):
         self._run("egpt_add_layernorm", h.data_ptr(), self._ptr(delta), splits, t, self._ptr(rows), weight.data_ptr(),
                   self._ptr(bias), float(eps), out.data_ptr(), n, hidden, dt, self._stream())
 
-    def normed_pair_mean(self, a, b, bias_a, bias_b, weight_a, weight_b, eps, factor):
-        """float32 [1, T, H]: factor * (rmsnorm(a + bias_a) * weight_a + rmsnorm(b + bias_b) * weight_b); a and b are
-        products (act [T, H] or float32 partial sums [S, T, H])."""
-        dt = self._act(weight_a, "weight_a")
+    def normed_pair_mean(self, a, b, bias_a, bias_b, weight_a, weight_b, eps, factor, factor_b=None, act_dtype=None):
+        """float32 [1, T, H]: factor * rmsnorm(a + bias_a) * weight_a + factor_b * rmsnorm(b + bias_b) * weight_b (factor_b
+        None: factor); a and b are products (act [T, H] or float32 partial sums [S, T, H]).  Without weights (both None;
+        act_dtype then names the products' type) nothing is normed: factor * (a + bias_a) + factor_b * (b + bias_b)."""
+        if (weight_a is None) != (weight_b is None):
+            raise ValueError("both branches are normed or neither")
+        ref = weight_a.dtype if weight_a is not None else act_dtype
+        if ref not in _DT:
+            raise TypeError("the products' type must be float32 or bfloat16")
+        dt = _DT[ref]
         t, hidden = a.shape[-2], a.shape[-1]
-        sa = self._product(a, "a", weight_a.dtype, t, hidden)
-        sb = self._product(b, "b", weight_a.dtype, t, hidden)
+        sa = self._product(a, "a", ref, t, hidden)
+        sb = self._product(b, "b", ref, t, hidden)
         for name, w in (("weight_a", weight_a), ("weight_b", weight_b), ("bias_a", bias_a), ("bias_b", bias_b)):
             if w is not None:
-                self._need(w, name, weight_a.dtype, (hidden,))
+                self._need(w, name, ref, (hidden,))
         out = torch.empty((1, t, hidden), dtype=_F32, device=a.device)
         self._run("egpt_normed_pair_mean", a.data_ptr(), sa, b.data_ptr(), sb, self._ptr(bias_a), self._ptr(bias_b),
-                  weight_a.data_ptr(), weight_b.data_ptr(), float(eps), float(factor), out.data_ptr(), t, hidden, dt,
-                  self._stream())
+                  self._ptr(weight_a), self._ptr(weight_b), float(eps), float(factor),
+                  float(factor if factor_b is None else factor_b), out.data_ptr(), t, hidden, dt, self._stream())
         return out
 
     def embed_positions(self, token_ids, positions, table, pos_table, out):
@@ -1115,9 +1148,12 @@ class HipKernels(KernelBackend):
         self._run("egpt_ff_activation", z.data_ptr(), splits, int(width), int(cols), modes[mode],
                   self._ptr(coef) if mode == "polynorm" else None, float(eps), int(gate_col), out.data_ptr(), t, dt, self._stream())
 
-    def tanh_cap(self, x, cap):
+    def tanh_cap(self, x, cap, scale=1.0):
+        """x <- x * scale, then x <- cap * tanh(x / cap) (cap None: the factor alone), in place."""
         self._need(x, "x", _F32)
-        self._run("egpt_tanh_cap", x.data_ptr(), float(cap), x.numel(), self._stream())
+        if cap is not None and not cap > 0:
+            raise ValueError(f"a cap ({cap}) must be positive")
+        self._run("egpt_tanh_cap", x.data_ptr(), float(scale), 0.0 if cap is None else float(cap), x.numel(), self._stream())
 
     def whole_norm_store(self, proj, bias, q_out, q_weight, k_weight, eps, positions, coef, every, slots, k_cache, v_cache,
                          nq, nkv, dk, dv, page_size):
@@ -1146,10 +1182,20 @@ class HipKernels(KernelBackend):
                   int(every), self._ptr(slots), self._ptr(k_cache) if slots is not None else None,
                   self._ptr(v_cache) if slots is not None else None, t, nq, nkv, dk, dv, page_size, dt, self._stream())
 
-    def head_norm_gate(self, x, weight, eps, gate, gate_offset, out, heads, dv):
+    def head_norm_gate(self, x, weight, eps, gate, gate_offset, out, heads, dv, gate_act="silu", x_width=None, x_act=None):
+        """x: float32 [T, W] or float32 partial sums [S, T, W], or (x_act given) a product of that activation type; its
+        rows are W = x_width values wide (heads * dv unless given) and the heads stand first.  gate_act: 'silu',
+        'sigmoid', or 'factor' (the gate's columns are multiplied in as they are)."""
         t = out.shape[0]
         dt = self._act(out, "out")
-        x_splits = self._product(x, "x", _F32, t, heads * dv)
+        acts = {"silu": 0, "sigmoid": 1, "factor": 2}
+        if gate_act not in acts:
+            raise ValueError(f"unknown gate activation '{gate_act}' (silu, sigmoid, factor)")
+        xw = heads * dv if x_width is None else int(x_width)
+        if xw < heads * dv:
+            raise ValueError(f"rows of {xw} values cannot hold {heads} heads of {dv}")
+        is_act = x.dim() == 2 and x_act is not None and x.dtype != _F32
+        x_splits = self._product(x, "x", x.dtype if is_act else _F32, t, xw)
         self._need(out, "out", None, (t, heads * dv))
         self._need(weight, "weight", out.dtype, (dv,))
         width, splits = 0, 0
@@ -1158,11 +1204,15 @@ class HipKernels(KernelBackend):
             splits = self._product(gate, "gate", out.dtype, t, width)
             if gate_offset < 0 or gate_offset + heads * dv > width:
                 raise ValueError(f"gate columns {gate_offset}..{gate_offset + heads * dv} lie outside rows of {width} values")
-        self._run("egpt_head_norm_gate", x.data_ptr(), x_splits, weight.data_ptr(), float(eps), self._ptr(gate), splits, int(width),
-                  int(gate_offset), out.data_ptr(), t, heads, dv, dt, self._stream())
+        self._run("egpt_head_norm_gate", x.data_ptr(), x_splits, 1 if is_act else 0, xw, weight.data_ptr(), float(eps),
+                  self._ptr(gate), splits, int(width), int(gate_offset), acts[gate_act], out.data_ptr(), t, heads, dv, dt,
+                  self._stream())
 
     # ------------------------------------------------------------------ a decaying matrix state per head
-    def channel_decay(self, low, low_offset, rank, w, bias, tau):
+    def channel_decay(self, low, low_offset, rank, w, bias, tau, rates=None, negate=False):
+        """float32 [T, C]: sigmoid(z)^(1 / tau) with z = low[:, low_offset : low_offset + rank] w^T + bias; rates float32 [C]
+        gives every channel an exponent of its own in place of 1 / tau, and negate takes -z for z, so that both together
+        are exp(-rates * softplus(z))."""
         t, width = low.shape[-2], low.shape[-1]
         dt = self._act(w, "w")
         channels = w.shape[0]
@@ -1172,9 +1222,12 @@ class HipKernels(KernelBackend):
         splits = self._product(low, "low", w.dtype, t, width)
         if low_offset < 0 or low_offset + rank > width:
             raise ValueError(f"columns {low_offset}..{low_offset + rank} lie outside rows of {width} values")
+        if rates is not None:
+            self._need(rates, "rates", _F32, (channels,))
         out = torch.empty((t, channels), dtype=_F32, device=w.device)
         self._run("egpt_channel_decay", low.data_ptr(), splits, int(width), int(low_offset), int(rank), w.data_ptr(),
-                  self._ptr(bias), float(tau), out.data_ptr(), t, channels, dt, self._stream())
+                  self._ptr(bias), float(tau), self._ptr(rates), 1 if negate else 0, out.data_ptr(), t, channels, dt,
+                  self._stream())
         return out
 
     def bounded_gate(self, z, z_offset, channels, bias, lower):
@@ -1196,13 +1249,20 @@ class HipKernels(KernelBackend):
         return out
 
     def decayed_state_scan(self, proj, act_dtype, q_offset, k_offset, v_offset, q_scale, decay, states, slots, fresh, q_start,
-                           q_len, heads, dk, dv, q_silu=False, tied_keys=False):
+                           q_len, heads, dk, dv, q_silu=False, tied_keys=False, k_silu=False, v_silu=False, head_decay=None):
+        """k_silu, v_silu: keys and values pass SiLU on their way in, as queries do with q_silu; head_decay float32 [heads]:
+        one constant decay per head (decay is then None)."""
         t, width = proj.shape[-2], proj.shape[-1]
         if act_dtype not in _DT:
             raise TypeError("act_dtype must be float32 or bfloat16")
         splits = self._product(proj, "proj", act_dtype, t, width)
         b = q_start.shape[0]
-        self._need(decay, "decay", _F32, (t, heads * dk))
+        if head_decay is not None:
+            self._need(head_decay, "head_decay", _F32, (heads,))
+            if decay is not None or tied_keys:
+                raise ValueError("a constant decay per head takes the place of the decays per token, and no keys are tied to it")
+        else:
+            self._need(decay, "decay", _F32, (t, heads * dk))
         self._need(states, "states", _F32)
         if states.dim() != 4 or tuple(states.shape[1:]) != (heads, dk, dv):
             raise ValueError(f"states must be [slots, {heads}, {dk}, {dv}], got {tuple(states.shape)}")
@@ -1214,11 +1274,79 @@ class HipKernels(KernelBackend):
         for off, n in ((q_offset, heads * dk), (None if tied_keys else k_offset, heads * dk), (v_offset, heads * dv)):
             if off is not None and (off < 0 or off + n > width):
                 raise ValueError(f"columns {off}..{off + n} lie outside rows of {width} values")
-        out = torch.empty((self.lib.egpt_scan_key_splits(dk), t, heads * dv), dtype=_F32, device=decay.device)
+        out = torch.empty((self.lib.egpt_scan_key_splits(dk), t, heads * dv), dtype=_F32, device=states.device)
         self._run("egpt_decayed_state_scan", proj.data_ptr(), splits, int(width), int(q_offset), 0 if tied_keys else int(k_offset), int(v_offset),
-                  float(q_scale), decay.data_ptr(), states.data_ptr(), slots.data_ptr(), self._ptr(fresh), q_start.data_ptr(),
+                  float(q_scale), self._ptr(decay), states.data_ptr(), slots.data_ptr(), self._ptr(fresh), q_start.data_ptr(),
                   q_len.data_ptr(), b, t, out.data_ptr(), heads, dk, dv, int(bool(q_silu)), int(bool(tied_keys)),
-                  _DT[act_dtype], self._stream())
+                  int(bool(k_silu)), int(bool(v_silu)), self._ptr(head_decay), _DT[act_dtype], self._stream())
+        return out
+
+    def _records(self, states, offset: int, floats: int):
+        """A part of every request's state record: states float32 [slots, N] -> (address of the first record's part, N)."""
+        self._need(states, "states", _F32)
+        if states.dim() != 2 or offset < 0 or offset + floats > states.shape[1]:
+            raise ValueError(f"state records of {tuple(states.shape)} floats cannot hold {floats} floats at place {offset}")
+        return states.data_ptr() + 4 * int(offset), int(states.shape[1])
+
+    def short_conv(self, proj, act_dtype, col0, conv_w, taps, unit_heads, unit_dim, scaled_heads, scale, unit_eps, sig_offset,
+                   n_sig, states, state_offset, slots, fresh, q_start, q_len, max_q_len):
+        """float32 [T, C + n_sig].  The columns col0 .. col0 + C of the product rows are the inputs of C short causal
+        convolutions over time (conv_w act [C, taps], the last column the current token's weight; the taps - 1 inputs
+        before a step's first token come from the request's record: states float32 [slots, N], the inputs at place
+        state_offset as [taps - 1, C]; zeros where fresh), then SiLU; the first unit_heads heads of unit_dim channels are
+        made unit vectors, x / sqrt(sum x^2 + unit_eps), the first scaled_heads of them times scale; behind the channels
+        comes the sigmoid of the columns sig_offset .. sig_offset + n_sig.  The records are brought up to date."""
+        t, width = proj.shape[-2], proj.shape[-1]
+        if act_dtype not in _DT:
+            raise TypeError("act_dtype must be float32 or bfloat16")
+        splits = self._product(proj, "proj", act_dtype, t, width)
+        channels = conv_w.shape[0]
+        self._need(conv_w, "conv_w", act_dtype, (channels, taps))
+        b = q_start.shape[0]
+        for name, v in (("slots", slots), ("q_start", q_start), ("q_len", q_len)):
+            self._need(v, name, _I32, (b,))
+        if fresh is not None:
+            self._need(fresh, "fresh", torch.bool, (b,))
+        if col0 < 0 or col0 + channels > width or (n_sig and (sig_offset < 0 or sig_offset + n_sig > width)):
+            raise ValueError(f"columns {col0}..{col0 + channels} or {sig_offset}..{sig_offset + n_sig} lie outside rows of {width} values")
+        if unit_heads * unit_dim > channels or not 0 <= scaled_heads <= unit_heads:
+            raise ValueError(f"{unit_heads} heads of {unit_dim} ({scaled_heads} scaled) do not fit {channels} channels")
+        base, stride = self._records(states, state_offset, (taps - 1) * channels)
+        out = torch.empty((t, channels + n_sig), dtype=_F32, device=states.device)
+        self._run("egpt_short_conv", proj.data_ptr(), splits, int(width), int(col0), conv_w.data_ptr(), int(taps), int(channels),
+                  int(unit_heads), int(unit_dim), int(scaled_heads), float(scale), float(unit_eps), int(sig_offset), int(n_sig),
+                  base, stride, slots.data_ptr(), self._ptr(fresh), q_start.data_ptr(), q_len.data_ptr(), b, int(max_q_len), t,
+                  out.data_ptr(), _DT[act_dtype], self._stream())
+        return out
+
+    def delta_rule_scan(self, ops, q_offset, k_offset, v_offset, beta_offset, decay, states, state_offset, slots, fresh, q_start,
+                        q_len, heads, kv_heads, dk, dv):
+        """float32 [1, T, heads * dv].  Per request and value head, token by token: S <- diag(decay_t) S; u = beta_t (v_t - S^T k_t);
+        S <- S + k_t u^T; o_t = S^T q_t.  ops float32 [T, W] holds queries and keys [kv_heads, dk], values [heads, dv] and beta
+        [heads] at their offsets (value head h reads query/key head h // (heads // kv_heads)); decay float32 [T, heads * dk];
+        the matrices [heads, dk, dv] lie at place state_offset of the records states float32 [slots, N]."""
+        self._need(ops, "ops", _F32)
+        if ops.dim() != 2:
+            raise ValueError("ops must be [tokens, values]")
+        t, width = ops.shape
+        b = q_start.shape[0]
+        self._need(decay, "decay", _F32, (t, heads * dk))
+        for name, v in (("slots", slots), ("q_start", q_start), ("q_len", q_len)):
+            self._need(v, name, _I32, (b,))
+        if fresh is not None:
+            self._need(fresh, "fresh", torch.bool, (b,))
+        if heads % kv_heads:
+            raise ValueError(f"heads ({heads}) must be a multiple of kv_heads ({kv_heads})")
+        for off, n in ((q_offset, kv_heads * dk), (k_offset, kv_heads * dk), (v_offset, heads * dv), (beta_offset, heads)):
+            if off < 0 or off + n > width:
+                raise ValueError(f"columns {off}..{off + n} lie outside rows of {width} values")
+        if dk > 1024:
+            raise ValueError(f"key size {dk} is not supported by the delta rule's scan (at most 1024)")
+        base, stride = self._records(states, state_offset, heads * dk * dv)
+        out = torch.empty((1, t, heads * dv), dtype=_F32, device=ops.device)
+        self._run("egpt_delta_rule_scan", ops.data_ptr(), int(width), int(q_offset), int(k_offset), int(v_offset), int(beta_offset),
+                  decay.data_ptr(), base, stride, slots.data_ptr(), self._ptr(fresh), q_start.data_ptr(), q_len.data_ptr(), b, t,
+                  out.data_ptr(), heads, kv_heads, dk, dv, self._stream())
         return out
 
     # ------------------------------------------------------------------ a mixture of experts

@@ -1,5 +1,5 @@
 from . import (attention, block, branch_mixers, depth_average, embedding, expert_mixture, feed_forward, gated_recurrence,  # noqa: F401
-               head_attention, local_attention, norm, position)      # (register the built-in parts)
+               head_attention, local_attention, norm, position, recurrent_mixers)      # (register the built-in parts)
 from .base import (
     BLOCKS,
     FEED_FORWARDS,

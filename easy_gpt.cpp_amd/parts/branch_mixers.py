@@ -13,8 +13,9 @@ channel; a head's output is RMS-normed with a weight that the heads share and mu
 float32, one record per request (`state_need`), and a step walks its tokens in order, so a prompt may be cut anywhere.
 
 `SideBySide`: two mixers that read the same input; each output is RMS-normed over the model width with a weight of
-its own, and the result is `factor` times their sum.  A branch hands over its output product unrounded (float32
-partial sums) with the bias that the product still lacks, and the join adds, norms and sums in float32.
+its own, and the result is `factor` times their sum; or, without norms, the result is the sum of the two outputs with
+a constant factor each.  A branch hands over its output product unrounded (float32 partial sums) with the bias that
+the product still lacks, and the join adds, norms and sums in float32.
 """
 from __future__ import annotations
 
@@ -197,11 +198,17 @@ class GatedLinearAttention(_Branch):
 
 class SideBySide(Mixer):
     def __init__(self, prefix: str, hidden_size: int, left: PartSpec, right: PartSpec, eps: float, factor: float = 0.5,
-                 names: dict | None = None):
-        """left, right: the two branches (mixers that offer `branch`); names: the weights of the two output norms
-        behind `prefix`."""
+                 names: dict | None = None, join: str = "normed_mean", factors: tuple | None = None):
+        """left, right: the two branches (mixers that offer `branch`).  join 'normed_mean': each output is RMS-normed
+        over the width with a weight of its own (names: those weights behind `prefix`) and the result is `factor` times
+        their sum; join 'weighted_sum': the result is factors[0] * left + factors[1] * right, no norms, no weights."""
+        if join not in ("normed_mean", "weighted_sum"):
+            raise ValueError(f"unknown join '{join}' of two mixers side by side (normed_mean, weighted_sum)")
+        if join == "weighted_sum" and (factors is None or len(factors) != 2):
+            raise ValueError("the join 'weighted_sum' takes factors=(left, right)")
         self.prefix, self.hidden_size = prefix, int(hidden_size)
-        self.eps, self.factor = float(eps), float(factor)
+        self.eps, self.factor, self.join = float(eps), float(factor), join
+        self.factors = (float(factors[0]), float(factors[1])) if join == "weighted_sum" else None
         self.branches = [make_part("mixer", left, hidden_size=hidden_size), make_part("mixer", right, hidden_size=hidden_size)]
         for b in self.branches:
             if not hasattr(b, "branch"):
@@ -222,18 +229,24 @@ class SideBySide(Mixer):
     def param_specs(self):
         h = self.hidden_size
         specs = [s for b in self.branches for s in b.param_specs()]
+        if self.join == "weighted_sum":
+            return specs
         return specs + [ParamSpec(self.prefix + self.names["left_out"], (h,), role="norm_scale"),
                         ParamSpec(self.prefix + self.names["right_out"], (h,), role="norm_scale")]
 
     def load(self, get, dtype, device):
         for b in self.branches:
             b.load(get, dtype, device)
-        self.out_weights = [self._to(get(self.prefix + self.names[x]), "compute", dtype, device) for x in ("left_out", "right_out")]
+        if self.join == "normed_mean":
+            self.out_weights = [self._to(get(self.prefix + self.names[x]), "compute", dtype, device) for x in ("left_out", "right_out")]
 
     def forward(self, x, ctx, cache, state=None):
         outs = [b.branch(x, ctx, cache if b.cache_need() is not None else None, state if b.state_need() is not None else None)
                 for b in self.branches]
         (a, bias_a), (b, bias_b) = outs
+        if self.join == "weighted_sum":
+            return kernels.backend().normed_pair_mean(a, b, bias_a, bias_b, None, None, self.eps, self.factors[0],
+                                                      factor_b=self.factors[1], act_dtype=x.dtype)
         return kernels.backend().normed_pair_mean(a, b, bias_a, bias_b, self.out_weights[0], self.out_weights[1], self.eps,
                                                   self.factor)
 

@@ -118,9 +118,10 @@ class LinearHead(OutputHead):
     graph_safe = True
 
     def __init__(self, prefix: str, hidden_size: int, vocab_size: int, tied: bool, name: str = "weight",
-                 softcap: float | None = None):
-        """softcap c: logits <- c * tanh(logits / c) (None: the product as it is)."""
+                 softcap: float | None = None, scale: float | None = None):
+        """scale s: logits <- s * logits; softcap c: then logits <- c * tanh(logits / c) (None: not)."""
         self.softcap = float(softcap) if softcap else None
+        self.scale = float(scale) if scale is not None and float(scale) != 1.0 else None
         self.prefix = prefix
         self.hidden_size = int(hidden_size)
         self.vocab_size = int(vocab_size)
@@ -146,8 +147,8 @@ class LinearHead(OutputHead):
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         out = torch.empty((x.shape[0], self.vocab_size), dtype=torch.float32, device=x.device)
         kernels.backend().linear(x, self.weight, None, out)
-        if self.softcap is not None:
-            kernels.backend().tanh_cap(out, self.softcap)
+        if self.softcap is not None or self.scale is not None:
+            kernels.backend().tanh_cap(out, self.softcap, scale=1.0 if self.scale is None else self.scale)
         return out
 
 
