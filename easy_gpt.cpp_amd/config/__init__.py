@@ -1,4 +1,5 @@
 from .base import ConfigError, KeyReader, read_json
+from .bubetar import BubetarConfig
 from .kezolix import KezolixConfig
 from .nebanex import NebanexConfig
 from .pekasun import PekasunConfig
@@ -15,6 +16,7 @@ from .registry import (
 
 __all__ = [
     "Architecture",
+    "BubetarConfig",
     "ConfigError",
     "KeyReader",
     "KezolixConfig",

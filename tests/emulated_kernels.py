@@ -118,18 +118,46 @@ class EmulatedKernels(KernelBackend):
             k_cache[page[i], :, off[i], :] = keys[i].to(k_cache.dtype)
             v_cache[page[i], :, :, off[i]] = values[i].to(v_cache.dtype)
 
+    @staticmethod
+    def _turn(a, cos_sin, magnitude, rotary_dim, pairing):
+        """a [T, heads, d]: the first rotary_dim places turned by the table's angles."""
+        a = a.clone()
+        if rotary_dim:
+            cs = cos_sin.to(F64) * magnitude
+            co, si = cs[:, None, :, 0], cs[:, None, :, 1]
+            if pairing == "interleaved":
+                u, w = a[..., 0:rotary_dim:2].clone(), a[..., 1:rotary_dim:2].clone()
+                a[..., 0:rotary_dim:2] = u * co - w * si
+                a[..., 1:rotary_dim:2] = w * co + u * si
+            else:
+                half = rotary_dim // 2
+                u, w = a[..., :half].clone(), a[..., half:rotary_dim].clone()
+                a[..., :half] = u * co - w * si
+                a[..., half:rotary_dim] = w * co + u * si
+        return a
+
     def head_norm_store(self, proj, q_out, q_weight, k_weight, eps, norm_values, slots, k_cache, v_cache, nq, nkv, dk, dv,
-                        page_size):
+                        page_size, row_width=None, cos_sin=None, rotary_dim=0, pairing="half", magnitude=1.0, norm_plain=False,
+                        norm_after_rotation=False, values_are_keys=False):
         x = _whole(proj).to(F64)
         t = x.shape[0]
         unit = lambda a: a / torch.sqrt((a * a).mean(-1, keepdim=True) + eps)
         q = x[:, : nq * dk].view(t, nq, dk)
         k = x[:, nq * dk : (nq + nkv) * dk].view(t, nkv, dk)
-        v = x[:, (nq + nkv) * dk :].view(t, nkv, dv)
+        v = k.clone() if values_are_keys else x[:, (nq + nkv) * dk : (nq + nkv) * dk + nkv * dv].view(t, nkv, dv)
+        turn = lambda a: self._turn(a, cos_sin, magnitude, rotary_dim, pairing)
+        if norm_after_rotation:
+            q, k = turn(q), turn(k)
         if q_weight is not None:
             q = unit(q) * q_weight.to(F64)
+        elif norm_plain:
+            q = unit(q)
         if k_weight is not None:
             k = unit(k) * k_weight.to(F64)
+        elif norm_plain:
+            k = unit(k)
+        if not norm_after_rotation:
+            q, k = turn(q), turn(k)
         if norm_values:
             v = unit(v)
         q_out.copy_(q.reshape(t, nq * dk).to(q_out.dtype))
@@ -137,11 +165,11 @@ class EmulatedKernels(KernelBackend):
             self._store(k_cache, v_cache, slots, page_size, k, v)
 
     def latent_prep(self, proj, q_plain, q_full, c_weight, eps, cos_sin, magnitude, rotary_dim, slots, k_cache, v_cache,
-                    nq, dim, rot, rank, page_size):
+                    nq, dim, rot, rank, page_size, queries=None, lead_width=None):
         x = _whole(proj).to(F64)
         t = x.shape[0]
-        q = x[:, : nq * (dim + rot)].view(t, nq, dim + rot)
-        base = nq * (dim + rot)
+        q = (x if queries is None else _whole(queries).to(F64))[:, : nq * (dim + rot)].view(t, nq, dim + rot)
+        base = nq * (dim + rot) if queries is None else lead_width
         c, shared = x[:, base : base + rank], x[:, base + rank : base + rank + rot]
         c = c / torch.sqrt((c * c).mean(-1, keepdim=True) + eps) * c_weight.to(F64)
 
@@ -223,17 +251,21 @@ class EmulatedKernels(KernelBackend):
         y = (x - mu) / torch.sqrt(((x - mu) ** 2).mean(-1, keepdim=True) + eps) * weight.to(F64)
         out.copy_((y if bias is None else y + bias.to(F64)).to(out.dtype))
 
-    def normed_pair_mean(self, a, b, bias_a, bias_b, weight_a, weight_b, eps, factor):
+    def normed_pair_mean(self, a, b, bias_a, bias_b, weight_a, weight_b, eps, factor, factor_b=None, act_dtype=None):
         def normed(x, bias, w):
             x = _whole(x).to(F64)
             if bias is not None:
                 x = x + bias.to(F64)
+            if w is None:
+                return x
             return x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps) * w.to(F64)
 
-        return (factor * (normed(a, bias_a, weight_a) + normed(b, bias_b, weight_b))).to(torch.float32)[None]
+        fb = factor if factor_b is None else factor_b
+        return (factor * normed(a, bias_a, weight_a) + fb * normed(b, bias_b, weight_b)).to(torch.float32)[None]
 
-    def tanh_cap(self, x, cap):
-        x.copy_((cap * torch.tanh(x.to(F64) / cap)).to(x.dtype))
+    def tanh_cap(self, x, cap, scale=1.0):
+        y = x.to(F64) * scale
+        x.copy_((y if cap is None else cap * torch.tanh(y / cap)).to(x.dtype))
 
     def whole_norm_store(self, proj, bias, q_out, q_weight, k_weight, eps, positions, coef, every, slots, k_cache, v_cache,
                          nq, nkv, dk, dv, page_size):
@@ -253,21 +285,24 @@ class EmulatedKernels(KernelBackend):
         if slots is not None:
             self._store(k_cache, v_cache, slots, page_size, k.reshape(t, nkv, dk), v.reshape(t, nkv, dv))
 
-    def head_norm_gate(self, x, weight, eps, gate, gate_offset, out, heads, dv):
+    def head_norm_gate(self, x, weight, eps, gate, gate_offset, out, heads, dv, gate_act="silu", x_width=None, x_act=None):
         t = out.shape[0]
-        xx = _whole(x).to(F64).view(t, heads, dv)
+        xx = _whole(x).to(F64)[:, : heads * dv].reshape(t, heads, dv)
         xx = xx / torch.sqrt((xx * xx).mean(-1, keepdim=True) + eps) * weight.to(F64)
         if gate is None:
             out.copy_(xx.reshape(t, heads * dv).to(out.dtype))
             return
         g = _whole(gate)[:, gate_offset : gate_offset + heads * dv].to(F64)
-        out.copy_((xx.reshape(t, heads * dv) * g * torch.sigmoid(g)).to(out.dtype))
+        g = {"silu": g * torch.sigmoid(g), "sigmoid": torch.sigmoid(g), "factor": g}[gate_act]
+        out.copy_((xx.reshape(t, heads * dv) * g).to(out.dtype))
 
-    def channel_decay(self, low, low_offset, rank, w, bias, tau):
+    def channel_decay(self, low, low_offset, rank, w, bias, tau, rates=None, negate=False):
         z = _whole(low)[:, low_offset : low_offset + rank].to(F64) @ w.to(F64).T
         if bias is not None:
             z = z + bias.to(F64)
-        return (torch.sigmoid(z) ** (1.0 / tau)).to(torch.float32)
+        if negate:
+            z = -z
+        return (torch.sigmoid(z) ** (1.0 / tau if rates is None else rates.to(F64))).to(torch.float32)
 
     def bounded_gate(self, z, z_offset, channels, bias, lower):
         v = _whole(z)[:, z_offset : z_offset + channels].to(F64)
@@ -277,9 +312,11 @@ class EmulatedKernels(KernelBackend):
         return (low + (1.0 - low) * torch.sigmoid(v)).to(torch.float32)
 
     def decayed_state_scan(self, proj, act_dtype, q_offset, k_offset, v_offset, q_scale, decay, states, slots, fresh, q_start,
-                           q_len, heads, dk, dv, q_silu=False, tied_keys=False):
+                           q_len, heads, dk, dv, q_silu=False, tied_keys=False, k_silu=False, v_silu=False, head_decay=None):
         x = _whole(proj).to(F64)
         t = x.shape[0]
+        if head_decay is not None:
+            decay = head_decay.to(F64)[None, :, None].expand(t, heads, dk).reshape(t, heads * dk)
         out = torch.zeros((t, heads * dv), dtype=torch.float32)
         for b in range(q_start.shape[0]):
             s0, n, slot = int(q_start[b]), int(q_len[b]), int(slots[b])
@@ -291,10 +328,63 @@ class EmulatedKernels(KernelBackend):
                 q = (q * torch.sigmoid(q) if q_silu else q) * q_scale
                 k = 1.0 - decay[i].to(F64).view(heads, dk) if tied_keys else x[i, k_offset : k_offset + heads * dk].view(heads, dk)
                 v = x[i, v_offset : v_offset + heads * dv].view(heads, dv)
+                if k_silu:
+                    k = k * torch.sigmoid(k)
+                if v_silu:
+                    v = v * torch.sigmoid(v)
                 st = decay[i].to(F64).view(heads, dk)[:, :, None] * st + k[:, :, None] * v[:, None, :]
                 out[i] = torch.einsum("hkv,hk->hv", st, q).reshape(-1).to(torch.float32)
             states[slot] = st.to(states.dtype)
         return out
+
+    def short_conv(self, proj, act_dtype, col0, conv_w, taps, unit_heads, unit_dim, scaled_heads, scale, unit_eps, sig_offset,
+                   n_sig, states, state_offset, slots, fresh, q_start, q_len, max_q_len):
+        x = _whole(proj).to(F64)
+        t, c = x.shape[0], conv_w.shape[0]
+        w = conv_w.to(F64)
+        out = torch.zeros((t, c + n_sig), dtype=F64)
+        for b in range(q_start.shape[0]):
+            s0, n, slot = int(q_start[b]), int(q_len[b]), int(slots[b])
+            if n <= 0:
+                continue
+            record = states[slot, state_offset : state_offset + (taps - 1) * c].view(taps - 1, c)
+            before = torch.zeros((taps - 1, c), dtype=F64) if fresh is not None and bool(fresh[b]) else record.to(F64)
+            z = torch.cat([before, x[s0 : s0 + n, col0 : col0 + c]], dim=0)
+            y = sum(z[j : j + n] * w[:, j] for j in range(taps))
+            y = y * torch.sigmoid(y)
+            u = y[:, : unit_heads * unit_dim].reshape(n, unit_heads, unit_dim)
+            u = u / torch.sqrt((u * u).sum(-1, keepdim=True) + unit_eps)
+            u[:, :scaled_heads] = u[:, :scaled_heads] * scale
+            y[:, : unit_heads * unit_dim] = u.reshape(n, -1)
+            out[s0 : s0 + n, :c] = y
+            out[s0 : s0 + n, c:] = torch.sigmoid(x[s0 : s0 + n, sig_offset : sig_offset + n_sig])
+            if taps > 1:
+                record.copy_(z[n:].to(states.dtype))
+        return out.to(torch.float32)
+
+    def delta_rule_scan(self, ops, q_offset, k_offset, v_offset, beta_offset, decay, states, state_offset, slots, fresh, q_start,
+                        q_len, heads, kv_heads, dk, dv):
+        x = ops.to(F64)
+        t = x.shape[0]
+        group = heads // kv_heads
+        out = torch.zeros((t, heads * dv), dtype=torch.float32)
+        for b in range(q_start.shape[0]):
+            s0, n, slot = int(q_start[b]), int(q_len[b]), int(slots[b])
+            if n <= 0:
+                continue
+            record = states[slot, state_offset : state_offset + heads * dk * dv].view(heads, dk, dv)
+            st = torch.zeros((heads, dk, dv), dtype=F64) if fresh is not None and bool(fresh[b]) else record.to(F64)
+            for i in range(s0, s0 + n):
+                q = x[i, q_offset : q_offset + kv_heads * dk].view(kv_heads, dk).repeat_interleave(group, dim=0)
+                k = x[i, k_offset : k_offset + kv_heads * dk].view(kv_heads, dk).repeat_interleave(group, dim=0)
+                v = x[i, v_offset : v_offset + heads * dv].view(heads, dv)
+                beta = x[i, beta_offset : beta_offset + heads]
+                st = decay[i].to(F64).view(heads, dk)[:, :, None] * st
+                u = beta[:, None] * (v - torch.einsum("hkv,hk->hv", st, k))
+                st = st + k[:, :, None] * u[:, None, :]
+                out[i] = torch.einsum("hkv,hk->hv", st, q).reshape(-1).to(torch.float32)
+            record.copy_(st.to(states.dtype))
+        return out[None]
 
     def expert_mixture(self, x, router, router_bias, w_gate_up, w_down, top, gated=True, score_all=False, correction=None,
                        weight_scale=1.0):
