@@ -1,0 +1,323 @@
+"""Bubetar models on the GPU against the plain implementation (tests/plain_bubetar.py): every way of cutting requests
+into steps, in float32 and bfloat16, on small configurations that differ in every size; mixed batches with pages and
+state slots used again, with and without graphs; long decoding past every window with the states and the convolutions'
+inputs carried through; a key made to stand out so that the query at the window's last position sees it and the next
+one does not; a batch against each request alone; a slot that is used again; generation through the entry point and the
+command line; bin/trace_run as a subprocess."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import bubetar_models as BM
+import helpers as H
+import plain_bubetar as P
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+# as fractions of the largest logit: float32 is the rounding of float32 sums in another order; bfloat16 rounds
+# activations between kernels (never the stream, statistics, scores, decays, gates of the recurrences, unit norms, the
+# states or partial sums)
+TOL = {"float32": 3e-5, "bfloat16": 4e-2}
+# float32 holds at every row.  Under bfloat16, with attention drawn peaked, the rounding of one head's scores moves a
+# row in a hundred beyond the line (measured layer by layer on the deepest configuration: the median row is off by 1 %
+# of the scale, the worst of 300 by 4 to 5 %); such a row may lie beyond it, but none beyond 10 % (a key that is wrongly
+# seen moves rows by tenths of the scale, see the test of the loud key, which allows no such row)
+STRAY = {"float32": 0.0, "bfloat16": 0.01}
+NEVER = 0.1
+
+
+def match(rows, ref, dtype, what):
+    H.assert_rows_match(rows, ref, TOL[dtype], what, may_exceed=STRAY[dtype])
+    if STRAY[dtype]:
+        H.assert_rows_match(rows, ref, NEVER, what)
+
+
+# sizes of a real model's kind: heads of 128 and 64 (the matrix-core attention), a latent of 256 + 64, a delta rule with
+# states of 128 x 128 and two value heads per key head, a constant-decay state of 64 x 128, a window of 96
+CONFIG_E = BM.config(523, 256, 1e-6, [
+    BM.layer(BM.latent(4, 64, 64, 64, 96, 256, 0.09, 10000.0), 512),
+    BM.layer(BM.pair_2(BM.softmax_side(4, 2, 128, 128, 0.08, BM.rotation(1e6, 64, (8.0, 1.0, 4.0, 512)), 96), BM.delta_rule(2, 1, 128, 128, 4), 0.6, 1.1), 256),
+    BM.layer(BM.pair(BM.softmax_side(4, 1, 64, 128, 0.12, BM.rotation(10000.0, 32)), BM.constant_decay(2, 64, 128, (0.9, 0.999)), 1.2, 1.1), 384),
+], logit_scale=0.5, logit_softcap=15.0)
+ALL = dict(BM.CONFIGS, E=(CONFIG_E, 9))
+
+
+@pytest.fixture(scope="module")
+def models(tmp_path_factory):
+    return {name: BM.write_model(str(tmp_path_factory.mktemp(f"bubetar_{name}")), cfg, seed) for name, (cfg, seed) in ALL.items()}
+
+
+@pytest.fixture(autouse=True)
+def product_kernels():
+    from easy_gpt.cpp_amd import kernels
+
+    kernels.use_backend(None)
+    assert kernels.backend().name == "hip-gfx950"
+
+
+def engine(model_dir, dtype, **kw):
+    from easy_gpt.cpp_amd.engine import Engine
+
+    return Engine.from_dir(model_dir, dtype=dtype, device="cuda:0", **kw)
+
+
+def plain_rows(model_dir, reqs):
+    cfg, w = P.read_model(model_dir)
+    return {rid: P.forward(cfg, w, ids) for rid, ids in reqs.items()}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E", "F"])
+def test_every_cutting_agrees_with_plain(models, name, dtype):
+    cfg = ALL[name][0]
+    reqs = H.make_requests(cfg["vocab"], [150, 1, 47, 2, 96], seed=21)
+    ref = plain_rows(models[name], reqs)
+    cuttings = {"whole": H.trace_whole(reqs), "last decoded": H.trace_last_decoded(reqs, 40), "portions": H.trace_portions(reqs),
+                "mixed": H.trace_mixed(reqs, seed=5, decode_tail=20)}
+    for what, trace in cuttings.items():
+        for page_size in (16, 32, 48) if what == "whole" else (16, 48) if what == "mixed" else (16,):
+            need = H.max_live_tokens(trace, 64)
+            eng = engine(models[name], dtype, page_size=page_size, max_tokens=need, max_requests=4)
+            rows = H.replay(eng, trace)
+            assert len(rows) == sum(len(v) for v in reqs.values())
+            match(rows, ref, dtype, f"{name} {dtype} {what} pages of {page_size}")
+            assert eng.cache.free_pages() == [p.num_pages for p in eng.cache.pools]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("use_graphs", [True, False])
+def test_mixed_batches_with_pages_and_state_slots_used_again(models, dtype, use_graphs):
+    """Ten requests through four state slots and a pool that holds a third of their tokens; with the decode steps
+    replayed from graphs and kernel by kernel."""
+    name = "A"
+    cfg = ALL[name][0]
+    reqs = H.make_requests(cfg["vocab"], [70, 23, 110, 64, 37, 90, 5, 130, 49, 81], seed=33)
+    ref = plain_rows(models[name], reqs)
+    trace = H.trace_mixed(reqs, seed=9, decode_tail=24)
+    need = H.max_live_tokens(trace, 16)
+    eng = engine(models[name], dtype, page_size=16, max_tokens=need, max_requests=4, use_graphs=use_graphs)
+    rows = H.replay(eng, trace)
+    match(rows, ref, dtype, f"mixed {dtype}")
+    assert sum(-(-len(v) // 16) for v in reqs.values()) > 2 * max(p.num_pages for p in eng.cache.pools)
+    assert max(len(r["entries"]) for r in trace) == 4
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "C", "E"])
+def test_long_decoding_passes_every_window_and_carries_the_states(models, name, dtype):
+    """Three tokens as a prompt, then 337 one by one: windows of 12, 40, 64 and 96 tokens pass over decoded tokens alone,
+    and the matrices and the convolutions' inputs are carried through all of them."""
+    cfg = ALL[name][0]
+    reqs = H.make_requests(cfg["vocab"], [340], seed=44)
+    ref = plain_rows(models[name], reqs)
+    eng = engine(models[name], dtype, page_size=16, max_tokens=384, max_requests=2)
+    rows = H.replay(eng, H.trace_last_decoded(reqs, 337))
+    assert len(rows) == 340
+    match(rows, ref, dtype, f"long decoding {name} {dtype}")
+
+
+def _one_loud_key(cfg):
+    """Weights of a one-layer model whose window attention alone reaches the stream (the delta rule beside it has a
+    factor of zero) and in which token 7 has a key that the queries of token 9 weigh far above all others, and with it
+    a value of its own (the values are the keys as projected).  Channel 0 of the embedding marks token 7 and is all that
+    the last key feature of a head reads; channel 1 marks token 9 and is all that the last query feature reads (the last
+    features lie beyond the rotated ones, so the position does not turn them); the other features read the other
+    channels.  After the norm a query of token 9 is sqrt(dim) times the last unit vector, and so is a key of token 7."""
+
+    def change(w):
+        m = cfg["layers"][0]["mixer"]["left"]
+        g = torch.Generator().manual_seed(1)
+        w["embed"][:] = 0.3 * torch.randn(w["embed"].shape, generator=g)
+        w["embed"][:, :2] = 0.0
+        w["embed"][7, :] = 0.0
+        w["embed"][7, 0] = 6.0
+        w["embed"][9, :] = 0.0
+        w["embed"][9, 1] = 6.0
+        w["l0.norm1"][:] = 1.0
+        w["l0.mix.left.sink"][:] = 0.0
+        width = w["embed"].shape[1]
+        for name, heads, channel in (("k", m["kv_heads"], 0), ("q", m["heads"], 1)):
+            proj = w[f"l0.mix.left.{name}"]
+            proj[:] = torch.randn(proj.shape, generator=g) / width ** 0.5
+            proj[:, :2] = 0.0
+            for head in range(heads):
+                proj[(head + 1) * m["dim"] - 1, :] = 0.0
+                proj[(head + 1) * m["dim"] - 1, channel] = 1.0
+        for name in w:
+            w[name] = w[name].to(torch.bfloat16).to(torch.float32)
+
+    return change
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("window", [5, 64, 100])
+def test_a_loud_key_is_seen_to_the_windows_last_position_and_not_beyond(tmp_path, dtype, window):
+    """One key stands out at position `window`.  Asking tokens at the last position whose window holds it and at the
+    next one: as a whole prompt, in portions cut just before and just after the edge, and decoded one by one; against
+    the plain implementation, which also shows that the two rows differ by far more than the tolerance (so a window
+    that is one token off cannot pass)."""
+    side = BM.softmax_side(4, 2, 16, 16, 0.75, BM.rotation(10000.0, 8, (4.0, 1.0, 4.0, 32)), window)
+    cfg = BM.config(64, 48, 1e-5, [BM.layer(BM.pair_2(side, BM.delta_rule(2, 1, 8, 8, 3), 1.0, 0.0), None)])
+    path = BM.write_model(str(tmp_path / "m"), cfg, 3, change=_one_loud_key(cfg))
+    g = torch.Generator().manual_seed(window)
+    n = 3 * window + 2
+    tokens = torch.randint(10, 64, (n,), generator=g).tolist()
+    tokens[window] = 7
+    asks = [2 * window - 1, 2 * window, 2 * window - 2, 2 * window + 1, window - 1]
+    for p in asks:
+        tokens[p] = 9
+    c, w = P.read_model(path)
+    want = P.forward(c, w, tokens)
+    inside, outside = want[2 * window - 1], want[2 * window]
+    assert float((inside - outside).abs().max()) > 0.2 * float(want.abs().max())
+    reqs = {"r0": tokens}
+    cut = [("r0", a, b) for a, b in [(0, 2 * window - 1), (2 * window - 1, 2 * window + 1), (2 * window + 1, n)]]
+    portions = [H.step_record(s, [(rid, tokens[a:b], list(range(b - a)))], ["r0"] if b == n else []) for s, (rid, a, b) in enumerate(cut)]
+    for what, trace in [("whole", H.trace_whole(reqs)), ("decoded", H.trace_last_decoded(reqs, n - window - 1)), ("portions", portions),
+                        ("small portions", H.trace_portions(reqs))]:
+        eng = engine(path, dtype, page_size=16, max_tokens=-(-n // 64) * 64, max_requests=1)
+        H.assert_rows_match(H.replay(eng, trace), {"r0": want}, TOL[dtype], f"window {window} {dtype} {what}")
+
+
+def test_a_state_slot_that_is_used_again_starts_anew(models):
+    """A request that takes the slot of a finished one gets what it gets in a new engine, bit for bit (float32): neither
+    the matrices nor the convolutions' inputs of the request before reach it."""
+    from easy_gpt.cpp_amd.engine import StepEntry
+
+    name = "C"
+    cfg = ALL[name][0]
+    reqs = H.make_requests(cfg["vocab"], [60, 45], seed=12)
+    first = engine(models[name], "float32", page_size=16, max_tokens=128, max_requests=1)
+    first.add_request("b")
+    first.step([StepEntry("b", reqs["r1"][:20], [])])
+    alone = first.step([StepEntry("b", reqs["r1"][20:], [24])]).cpu().clone()
+    eng = engine(models[name], "float32", page_size=16, max_tokens=128, max_requests=1)
+    eng.add_request("a")
+    eng.step([StepEntry("a", reqs["r0"], [59])])
+    eng.finish("a")
+    eng.add_request("b")
+    assert eng.cache.requests["b"].slot == 0
+    eng.step([StepEntry("b", reqs["r1"][:20], [])])
+    again = eng.step([StepEntry("b", reqs["r1"][20:], [24])]).cpu()
+    assert torch.equal(again, alone)
+
+
+def test_a_batch_gives_each_request_what_it_gets_alone(models):
+    """float32: the logits of a request in a batch of unequal requests against the same request alone."""
+    name = "E"
+    cfg = ALL[name][0]
+    reqs = H.make_requests(cfg["vocab"], [90, 7, 33, 64], seed=55)
+    from easy_gpt.cpp_amd.engine import StepEntry
+
+    eng = engine(models[name], "float32", page_size=16, max_tokens=512, max_requests=4)
+    for rid in reqs:
+        eng.add_request(rid)
+    together = eng.step([StepEntry(rid, ids, [len(ids) - 1]) for rid, ids in reqs.items()]).cpu().clone()
+    scale = float(together.abs().max())
+    for i, (rid, ids) in enumerate(reqs.items()):
+        eng.finish(rid)
+        eng.add_request(rid)
+        alone = eng.step([StepEntry(rid, ids, [len(ids) - 1])]).cpu()
+        assert float((alone[0] - together[i]).abs().max()) <= 2e-6 * scale, rid
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_prompt_of_1500_tokens_in_one_step_then_single_tokens(models, dtype):
+    name = "C"
+    cfg = ALL[name][0]
+    reqs = H.make_requests(cfg["vocab"], [1510], seed=88)
+    ref = plain_rows(models[name], reqs)
+    eng = engine(models[name], dtype, page_size=16, max_tokens=1536, max_requests=1)
+    trace = H.trace_last_decoded(reqs, 10)
+    for rec in trace:                     # the logits of the last 200 tokens of the prompt and of the decoded ones
+        for e in rec["entries"]:
+            e["want"] = [i for i in e["want"] if len(e["tokens"]) == 1 or i >= len(e["tokens"]) - 200]
+    rows = H.replay(eng, trace)
+    assert len(rows) == 210
+    match(rows, ref, dtype, f"long prompt {dtype}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_greedy_generation_through_the_entry_point(models, dtype):
+    from easy_gpt.cpp_amd.generate import LLM
+
+    name = "A"
+    cfg = ALL[name][0]
+    prompts = list(H.make_requests(cfg["vocab"], [5, 40, 17, 1, 33, 8], seed=66).values())
+    llm = LLM(models[name], dtype=dtype, cache_tokens=1024, prefill_chunk=16)
+    outs = llm.generate(prompts, max_new_tokens=24, greedy=True, ignore_eos=True)
+    c, w = P.read_model(models[name])
+    for prompt, out in zip(prompts, outs):
+        assert len(out) == 24
+        logits = P.forward(c, w, prompt + out)
+        for i, tok in enumerate(out):
+            row = logits[len(prompt) + i - 1]
+            gap = float(row.max() - row[tok])
+            assert gap <= (1e-4 if dtype == "float32" else 5e-2) * float(row.abs().max()), (dtype, i, tok, gap)
+
+
+def test_generation_under_page_pressure_gives_the_tokens_of_a_run_with_room(models):
+    """Requests that are preempted and computed again get a state slot anew: the same tokens, bit for bit (float32)."""
+    from easy_gpt.cpp_amd.generate import LLM
+
+    name = "A"
+    cfg = ALL[name][0]
+    prompts = list(H.make_requests(cfg["vocab"], [50, 70, 30, 90, 20, 60, 45, 80], seed=67).values())
+    roomy = LLM(models[name], dtype="float32", cache_tokens=4096, prefill_chunk=32)
+    want = roomy.generate(prompts, max_new_tokens=40, greedy=True, ignore_eos=True)
+    tight = LLM(models[name], dtype="float32", cache_tokens=400, prefill_chunk=32)
+    got = tight.generate(prompts, max_new_tokens=40, greedy=True, ignore_eos=True)
+    assert got == want
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_as_a_subprocess(models, tmp_path, dtype):
+    name = "B"
+    cfg = ALL[name][0]
+    reqs = H.make_requests(cfg["vocab"], [70, 23, 110, 37, 55], seed=77)
+    ref = plain_rows(models[name], reqs)
+    trace = H.trace_mixed(reqs, seed=4, decode_tail=32, want_all=False)
+    out_dir = str(tmp_path / "out")
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", models[name], "--dtype", dtype, "--out", out_dir,
+           "--max-tokens", str(H.max_live_tokens(trace, 64))]
+    p = subprocess.Popen(cmd, stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True)
+    rows, fed = {}, {}
+    for rec in trace:
+        p.stdin.write(json.dumps(rec) + "\n")
+        p.stdin.flush()
+        assert p.stdout.readline().strip() == f"done {rec['step']}"
+        wanted = sum(len(e["want"]) for e in rec["entries"])
+        if wanted:
+            data = np.fromfile(os.path.join(out_dir, f"{rec['step']}.f32"), dtype="<f4").reshape(wanted, cfg["vocab"])
+            r = 0
+            for e in rec["entries"]:
+                for w in e["want"]:
+                    rows[(e["id"], fed.get(e["id"], 0) + w)] = torch.from_numpy(data[r].copy())
+                    r += 1
+        for e in rec["entries"]:
+            fed[e["id"]] = fed.get(e["id"], 0) + len(e["tokens"])
+    p.stdin.close()
+    assert p.wait(timeout=60) == 0
+    assert len(rows) > 60
+    match(rows, ref, dtype, f"trace_run {dtype}")
+
+
+def test_the_command_line_generates_with_a_bubetar_folder(models):
+    name = "A"
+    prompt = [5, 17, 3, 250, 9, 44, 1]
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "easy_llm"), "--model", models[name], "--dtype", "float32", "--greedy",
+           "--ignore-eos", "--max-new-tokens", "12"]
+    p = subprocess.run(cmd + [" ".join(map(str, prompt))], capture_output=True, text=True, timeout=110, cwd=ROOT)
+    assert p.returncode == 0, p.stderr[-2000:]
+    c, w = P.read_model(models[name])
+    out = [int(t) for t in p.stdout.split()]
+    assert len(out) == 12
+    logits = P.forward(c, w, prompt + out)
+    for i, tok in enumerate(out):
+        row = logits[len(prompt) + i - 1]
+        assert float(row.max() - row[tok]) <= 1e-4 * float(row.abs().max()), (i, tok)
