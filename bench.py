@@ -440,6 +440,36 @@ def kezolix_config(width, heads, kv_heads, hd, s_heads, s_dim, s_vdim, experts, 
             "residual_mult": 0.5, "layers": layers}
 
 
+# `--design bubetar`: the Bubetar design (latent attention with latent queries; attention with normed, rotated heads and
+# an output gate beside linear attention with a constant decay per head; window attention on its own keys with a sink
+# beside a gated delta rule with short convolutions; a layer norm before and behind every branch; a dense gated
+# feed-forward) beside the Nebanex model of the same sizes, whose layers also hold a softmax attention and a matrix state
+# side by side, and beside the Qwen2 model of the same width, heads and inner width.  The sizes are Nebanex's, the
+# feed-forward as wide as what a Nebanex token uses, the latents those of the Pekasun comparison; the layers: window
+# attention + delta rule, latent attention, gated attention + constant decay, latent attention.
+def bubetar_config(width, heads, kv_heads, hd, s_heads, s_dim, s_vdim, inner, rank, rot, window) -> dict:
+    ff = {"kind": "dense", "ff": inner}
+    latent = {"type": "latent_attention", "mlp": ff,
+              "mixer": {"heads": heads, "dim": hd, "rot_dim": rot, "vdim": hd, "q_rank": 3 * rank, "kv_rank": rank,
+                        "scale": (hd + rot) ** -0.5, "rot": {"base": 10000.0, "dims": rot}}}
+    gated = {"type": "parallel", "mlp": ff,
+             "mixer": {"left": {"heads": heads, "kv_heads": kv_heads, "dim": hd, "vdim": hd, "scale": hd ** -0.5,
+                                "rot": {"base": 10000.0, "dims": hd // 2}},
+                       "right": {"heads": s_heads, "dim": s_dim, "vdim": s_vdim,
+                                 "decay": [1.0 - 2.0 ** (-3 - 5 * h / s_heads) for h in range(s_heads)]},
+                       "left_scale": 1.0, "right_scale": 1.0}}
+    delta = {"type": "parallel_2", "mlp": ff,
+             "mixer": {"left": {"heads": heads, "kv_heads": kv_heads, "dim": hd, "vdim": hd, "scale": hd ** -0.5,
+                                "mask": {"size": window},
+                                "rot": {"base": 1000000.0, "dims": hd, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}},
+                       "right": {"heads": s_heads, "kv_heads": s_heads, "dim": s_dim, "vdim": s_vdim, "conv": 4},
+                       "left_scale": 1.0, "right_scale": 1.0}}
+    layers = [delta, latent, gated, latent]
+    assert len(layers) == DESIGN_LAYERS
+    return {"architecture": "Bubetar", "vocab": DESIGN_VOCAB, "width": width, "norm": {"eps": 1e-6}, "logit_scale": 0.5,
+            "logit_softcap": 30.0, "layers": layers}
+
+
 def design_models(design):
     """(label, {name: config}) for every size of the comparison, and how the sizes are named in the record."""
     if design == "pekasun":
@@ -447,6 +477,13 @@ def design_models(design):
         for s in DESIGN_SIZES:
             label, width, inner, heads, kv_heads, hd = s[:6]
             yield label, dict(zip(keys, s[1:])), pekasun_config(*s[1:]), (width, inner, heads, kv_heads, hd)
+    elif design == "bubetar":
+        keys = ("width", "heads", "kv_heads", "head", "state_heads", "state_key", "state_value", "inner", "latent", "rotated", "window")
+        for s, d in zip(NEBANEX_SIZES, DESIGN_SIZES):
+            label, width, heads, kv_heads, hd, s_heads, s_dim, s_vdim = s[:8]
+            inner = s[9] * s[10] + s[11]
+            sizes = (width, heads, kv_heads, hd, s_heads, s_dim, s_vdim, inner, d[6], d[7], d[8])
+            yield label, dict(zip(keys, sizes)), bubetar_config(*sizes), (width, inner, heads, kv_heads, hd)
     else:
         keys = ("width", "heads", "kv_heads", "head", "state_heads", "state_key", "state_value", "experts", "chosen",
                 "expert_inner", "shared_inner")
@@ -470,7 +507,7 @@ def design_comparison(args) -> dict:
         sizes[label] = named
         models = {
             design: design_cfg,
-            **({"nebanex": nebanex_config(*next(s for s in NEBANEX_SIZES if s[0] == label)[1:])} if design == "kezolix" else {}),
+            **({"nebanex": nebanex_config(*next(s for s in NEBANEX_SIZES if s[0] == label)[1:])} if design in ("kezolix", "bubetar") else {}),
             "qwen2": dict(QWEN25_05B, hidden_size=width, intermediate_size=inner, num_attention_heads=heads,
                           num_key_value_heads=kv_heads, head_dim=hd, num_hidden_layers=DESIGN_LAYERS, vocab_size=DESIGN_VOCAB,
                           tie_word_embeddings=False),
@@ -536,9 +573,9 @@ def main() -> int:
     ap.add_argument("--no-lookahead", action="store_true",
                     help="wait for a step's tokens on the host before the next step is launched (the scheduler with --serve, "
                          "the decode loop otherwise)")
-    ap.add_argument("--design", default=None, choices=["pekasun", "nebanex", "kezolix"],
+    ap.add_argument("--design", default=None, choices=["pekasun", "nebanex", "kezolix", "bubetar"],
                     help="instead of the record: prefill and decode of that design at a few layer sizes beside the Qwen2 "
-                         "model of equal sizes (kezolix: also beside the Nebanex model of equal sizes)")
+                         "model of equal sizes (kezolix, bubetar: also beside the Nebanex model of equal sizes)")
     ap.add_argument("--direct-loop", action="store_true",
                     help="decode with the engine's step function in a loop of the benchmark's own instead of Scheduler.step")
     args = ap.parse_args()

@@ -364,117 +364,188 @@ __global__ __launch_bounds__(256) void conv_carry_kernel(ProductView<T> proj, in
     }
 }
 
-// One workgroup per (request, head, 64 value channels); a lane is a column of the head's state S [dk][dv], and wavefront w
-// keeps the key channels w * DKR .. of that column in registers.  Per token: the column decays row by row, every wavefront
-// sums its rows' part of S^T k, the parts meet in LDS (two buffers in turn, so one barrier a token), u = beta (v - S^T k),
-// the rows take k u, and the wavefronts' parts of S^T q are kept for the end of the batch, where they are added in the
-// order of the wavefronts.  A batch of `tb` tokens' operands is staged in LDS.  Value head h reads the queries and keys of
-// head h / (heads / kv_heads).  ops rows hold queries, keys, values and beta (float32); decay is [tokens][heads * dk].
-template <int DKR>
-__global__ __launch_bounds__(1024) void delta_rule_scan_kernel(
+// The delta rule's scan.  A workgroup is one wavefront that owns 64 / SLICES columns of a head's state S [dk][dv]: its
+// lanes are columns x SLICES ranges of R key channels (SLICES a power of two, SLICES * R >= dk), a lane keeps its range of
+// its column in registers, and what has to be summed over the key channels (S^T k, S^T q and k . q) is summed over a
+// lane's rows and then across the slices with lane exchanges: no barrier and no trip through memory stands between two
+// tokens.  With S' = diag(g) S the token's output is S'^T q + (k . q) u, u = beta (v - S'^T k), so the sums are taken on
+// the decayed state before it is written, and the write S <- S' + k u^T is off the path to the next token's sums.  The
+// operands are staged in LDS a batch of TB tokens at a time (queries, keys and decays of the head, the wavefront's columns
+// of the values, beta) while the next batch's loads are in flight in registers, all of them issued together, and a token's
+// operands are read from LDS while the token before is computed; outputs leave through LDS, a batch at a time.  What
+// bounds a token is the vector arithmetic of a lane's rows (four operations a row) and what LDS returns for them (every lane
+// gets its copy of its slice's queries, keys and decays: one wavefront to a workgroup, so that wavefronts do not share a
+// CU's LDS while there are CUs to spare).  Value head h reads the queries and keys of head h / (heads / kv_heads).  ops rows
+// hold queries, keys, values and beta (float32); decay is [tokens][heads * dk].
+// The sum of v over the N neighbouring lanes that hold the slices of one column (N a power of two, lanes N * i ..), in every
+// one of them.  Within a row of 16 lanes the exchanges are operand modifiers of the additions themselves (pairs, quads,
+// then the mirrored half row and the mirrored row, which hold equal values by then); beyond a row they go through the
+// lane permute.
+template <int CTRL>
+__device__ __forceinline__ float lanes_add(float v) {
+    return v + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+template <int N>
+__device__ __forceinline__ float slices_sum(float v) {
+    if (N >= 2) v = lanes_add<0xB1>(v);          // quad_perm [1, 0, 3, 2]
+    if (N >= 4) v = lanes_add<0x4E>(v);          // quad_perm [2, 3, 0, 1]
+    if (N >= 8) v = lanes_add<0x141>(v);         // row_half_mirror
+    if (N >= 16) v = lanes_add<0x140>(v);        // row_mirror
+    if (N >= 32) v += __shfl_xor(v, 16, kWave);
+    if (N >= 64) v += __shfl_xor(v, 32, kWave);
+    return v;
+}
+
+template <int SLICES, int R>
+__global__ __launch_bounds__(64) void delta_rule_scan_kernel(
     const float* __restrict__ ops, int ops_width, int q_off, int k_off, int v_off, int beta_off, const float* __restrict__ decay,
     float* __restrict__ states, size_t state_stride, const int32_t* __restrict__ slots, const unsigned char* __restrict__ fresh,
     const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len, float* __restrict__ out, int heads, int kv_heads,
-    int dk, int dv, int tb) {
-    extern __shared__ __attribute__((aligned(16))) float scan_s[];
-    const int nw = blockDim.x / kWave, dkp = nw * DKR;
-    float* q_s = scan_s;
-    float* k_s = q_s + tb * dkp;
-    float* g_s = k_s + tb * dkp;
-    float* v_s = g_s + tb * dkp;
-    float* beta_s = v_s + tb * kScanCols;
-    float* part_s = beta_s + ((tb + 3) & ~3);
-    float* red_s = part_s + tb * nw * kScanCols;
-    const int b = blockIdx.x, h = blockIdx.y, col0 = blockIdx.z * kScanCols;
+    int dk, int dv) {
+    constexpr int THREADS = kWave, DKP = SLICES * R;
+    constexpr int COLS = kWave / SLICES, WG_COLS = COLS;
+    constexpr int WIDEST = DKP > WG_COLS ? DKP : WG_COLS;
+    constexpr int TB = 512 / WIDEST < 16 ? (512 / WIDEST < 1 ? 1 : 512 / WIDEST) : 16;      // tokens to a batch: about 512 values of an operand
+    constexpr int QKA = (TB * DKP + THREADS - 1) / THREADS;             // values of q (or k, or g) of a batch per thread
+    constexpr int VL = (TB * WG_COLS + THREADS - 1) / THREADS;          // values of v, and outputs, of a batch per thread
+    __shared__ __attribute__((aligned(16))) float q_s[TB * DKP];
+    __shared__ __attribute__((aligned(16))) float k_s[TB * DKP];
+    __shared__ __attribute__((aligned(16))) float g_s[TB * DKP];
+    __shared__ float v_s[TB * WG_COLS];
+    __shared__ float o_s[TB * WG_COLS];
+    __shared__ float beta_s[TB];
+    const int b = blockIdx.x, h = blockIdx.y, col0 = blockIdx.z * WG_COLS;
     const int n = q_len[b];
     if (n <= 0) return;
     const int t0 = q_start[b];
-    const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
-    const int j = col0 + lane;
+    const int tid = threadIdx.x, lane = tid;
+    const int sl = lane % SLICES, c = lane / SLICES;                     // this lane's slice of the key channels, and its column
+    const int j = col0 + c;
     const bool has_col = j < dv;
     const int kvh = h / (heads / kv_heads);
     float* state = states + static_cast<size_t>(slots[b]) * state_stride + static_cast<size_t>(h) * dk * dv;
     const bool anew = fresh != nullptr && fresh[b] != 0;
-    float s[DKR];
+    float s[R];
 #pragma unroll
-    for (int i = 0; i < DKR; ++i) {
-        const int r = wave * DKR + i;
+    for (int i = 0; i < R; ++i) {
+        const int r = sl * R + i;
         s[i] = (!anew && has_col && r < dk) ? state[static_cast<size_t>(r) * dv + j] : 0.f;
     }
-    const int threads = blockDim.x;
-    for (int base = 0; base < n; base += tb) {
-        const int count = min(tb, n - base);
-        __syncthreads();                              // the batch before is read, its parts are added
-        for (int idx = tid; idx < count * dkp; idx += threads) {
-            const int tt = idx / dkp, r = idx % dkp;
-            const size_t row = static_cast<size_t>(t0 + base + tt);
-            const bool valid = r < dk;
-            q_s[idx] = valid ? ops[row * ops_width + q_off + kvh * dk + r] : 0.f;
-            k_s[idx] = valid ? ops[row * ops_width + k_off + kvh * dk + r] : 0.f;
-            g_s[idx] = valid ? decay[row * heads * dk + static_cast<size_t>(h) * dk + r] : 0.f;
-        }
-        for (int idx = tid; idx < count * kScanCols; idx += threads) {
-            const int tt = idx / kScanCols, c = idx % kScanCols;
-            const size_t row = static_cast<size_t>(t0 + base + tt);
-            v_s[idx] = col0 + c < dv ? ops[row * ops_width + v_off + h * dv + col0 + c] : 0.f;
-        }
-        for (int idx = tid; idx < count; idx += threads)
-            beta_s[idx] = ops[static_cast<size_t>(t0 + base + idx) * ops_width + beta_off + h];
-        __syncthreads();
-        for (int tt = 0; tt < count; ++tt) {
-            const float4* g4 = reinterpret_cast<const float4*>(g_s + tt * dkp + wave * DKR);
-            const float4* k4 = reinterpret_cast<const float4*>(k_s + tt * dkp + wave * DKR);
-            const float4* q4 = reinterpret_cast<const float4*>(q_s + tt * dkp + wave * DKR);
-            float kk[DKR];
-            float p = 0.f;
+    float rq[QKA], rk[QKA], rg[QKA], rv[VL], rbeta = 0.f;
+    auto fetch = [&](int base) {
+        const int count = min(TB, n - base);
 #pragma unroll
-            for (int i = 0; i < DKR / 4; ++i) {
-                const float4 g = g4[i], k = k4[i];
-                kk[4 * i] = k.x, kk[4 * i + 1] = k.y, kk[4 * i + 2] = k.z, kk[4 * i + 3] = k.w;
-                s[4 * i] *= g.x, s[4 * i + 1] *= g.y, s[4 * i + 2] *= g.z, s[4 * i + 3] *= g.w;
-                p = fmaf(s[4 * i], k.x, p);
-                p = fmaf(s[4 * i + 1], k.y, p);
-                p = fmaf(s[4 * i + 2], k.z, p);
-                p = fmaf(s[4 * i + 3], k.w, p);
+        for (int u = 0; u < QKA; ++u) {
+            const int idx = tid + u * THREADS;
+            const int tt = idx / DKP, r = idx % DKP;
+            rq[u] = rk[u] = rg[u] = 0.f;
+            if (tt < count && r < dk) {                                  // (tt < count <= TB bounds idx as well)
+                const size_t row = static_cast<size_t>(t0 + base + tt);
+                rq[u] = ops[row * ops_width + q_off + kvh * dk + r];
+                rk[u] = ops[row * ops_width + k_off + kvh * dk + r];
+                rg[u] = decay[row * heads * dk + static_cast<size_t>(h) * dk + r];
             }
-            float* red = red_s + (tt & 1) * nw * kScanCols;
-            red[wave * kScanCols + lane] = p;
-            __syncthreads();
-            float total = 0.f;
-            for (int w = 0; w < nw; ++w) total += red[w * kScanCols + lane];
-            const float u = beta_s[tt] * (v_s[tt * kScanCols + lane] - total);
-            float po = 0.f;
+        }
 #pragma unroll
-            for (int i = 0; i < DKR / 4; ++i) {
-                const float4 q = q4[i];
-                s[4 * i] = fmaf(kk[4 * i], u, s[4 * i]);
-                s[4 * i + 1] = fmaf(kk[4 * i + 1], u, s[4 * i + 1]);
-                s[4 * i + 2] = fmaf(kk[4 * i + 2], u, s[4 * i + 2]);
-                s[4 * i + 3] = fmaf(kk[4 * i + 3], u, s[4 * i + 3]);
-                po = fmaf(s[4 * i], q.x, po);
-                po = fmaf(s[4 * i + 1], q.y, po);
-                po = fmaf(s[4 * i + 2], q.z, po);
-                po = fmaf(s[4 * i + 3], q.w, po);
+        for (int u = 0; u < VL; ++u) {
+            const int idx = tid + u * THREADS;
+            const int tt = idx / WG_COLS, cc = idx % WG_COLS;
+            rv[u] = 0.f;
+            if (tt < count && col0 + cc < dv)
+                rv[u] = ops[static_cast<size_t>(t0 + base + tt) * ops_width + v_off + h * dv + col0 + cc];
+        }
+        rbeta = tid < count ? ops[static_cast<size_t>(t0 + base + tid) * ops_width + beta_off + h] : 0.f;      // (TB <= 16 < 64)
+    };
+    fetch(0);
+    for (int base = 0; base < n; base += TB) {
+        const int count = min(TB, n - base);
+        __syncthreads();                              // the batch before is read
+#pragma unroll
+        for (int u = 0; u < QKA; ++u) {
+            if (tid + u * THREADS < TB * DKP) {
+                q_s[tid + u * THREADS] = rq[u];
+                k_s[tid + u * THREADS] = rk[u];
+                g_s[tid + u * THREADS] = rg[u];
             }
-            part_s[(tt * nw + wave) * kScanCols + lane] = po;
+        }
+#pragma unroll
+        for (int u = 0; u < VL; ++u)
+            if (tid + u * THREADS < TB * WG_COLS) v_s[tid + u * THREADS] = rv[u];
+        if (tid < TB) beta_s[tid] = rbeta;
+        __syncthreads();
+        if (base + TB < n) fetch(base + TB);
+        // (a token's operands are read from LDS while the token before is computed: two sets of registers in turn)
+        float4 ga[R / 4], ka[R / 4], qa[R / 4], gb[R / 4], kb[R / 4], qb[R / 4];
+        float va, ba, vb, bb;
+        auto read = [&](int tt, float4* g, float4* k, float4* q, float& vj, float& beta) {
+            const int at = tt < TB ? tt : TB - 1;                        // (behind the batch's last token: read and not used)
+#pragma unroll
+            for (int i = 0; i < R / 4; ++i) {
+                g[i] = reinterpret_cast<const float4*>(g_s + at * DKP + sl * R)[i];
+                k[i] = reinterpret_cast<const float4*>(k_s + at * DKP + sl * R)[i];
+                q[i] = reinterpret_cast<const float4*>(q_s + at * DKP + sl * R)[i];
+            }
+            vj = v_s[at * WG_COLS + c];
+            beta = beta_s[at];
+        };
+        auto token = [&](int tt, const float4* g, const float4* k, const float4* q, float vj, float beta) {
+            float pk[4] = {0.f, 0.f, 0.f, 0.f}, pq[4] = {0.f, 0.f, 0.f, 0.f}, kq[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int i = 0; i < R / 4; ++i) {
+                s[4 * i] *= g[i].x, s[4 * i + 1] *= g[i].y, s[4 * i + 2] *= g[i].z, s[4 * i + 3] *= g[i].w;
+                pk[0] = fmaf(s[4 * i], k[i].x, pk[0]), pk[1] = fmaf(s[4 * i + 1], k[i].y, pk[1]);
+                pk[2] = fmaf(s[4 * i + 2], k[i].z, pk[2]), pk[3] = fmaf(s[4 * i + 3], k[i].w, pk[3]);
+                pq[0] = fmaf(s[4 * i], q[i].x, pq[0]), pq[1] = fmaf(s[4 * i + 1], q[i].y, pq[1]);
+                pq[2] = fmaf(s[4 * i + 2], q[i].z, pq[2]), pq[3] = fmaf(s[4 * i + 3], q[i].w, pq[3]);
+                kq[0] = fmaf(k[i].x, q[i].x, kq[0]), kq[1] = fmaf(k[i].y, q[i].y, kq[1]);
+                kq[2] = fmaf(k[i].z, q[i].z, kq[2]), kq[3] = fmaf(k[i].w, q[i].w, kq[3]);
+            }
+            const float sk = slices_sum<SLICES>((pk[0] + pk[1]) + (pk[2] + pk[3]));
+            const float sq = slices_sum<SLICES>((pq[0] + pq[1]) + (pq[2] + pq[3]));
+            const float skq = slices_sum<SLICES>((kq[0] + kq[1]) + (kq[2] + kq[3]));
+            const float u = beta * (vj - sk);
+            if (sl == 0) o_s[tt * WG_COLS + c] = fmaf(skq, u, sq);
+#pragma unroll
+            for (int i = 0; i < R / 4; ++i) {
+                s[4 * i] = fmaf(k[i].x, u, s[4 * i]), s[4 * i + 1] = fmaf(k[i].y, u, s[4 * i + 1]);
+                s[4 * i + 2] = fmaf(k[i].z, u, s[4 * i + 2]), s[4 * i + 3] = fmaf(k[i].w, u, s[4 * i + 3]);
+            }
+        };
+        read(0, ga, ka, qa, va, ba);
+        for (int tt = 0; tt < count; tt += 2) {
+            read(tt + 1, gb, kb, qb, vb, bb);
+            token(tt, ga, ka, qa, va, ba);
+            if (tt + 1 < count) {
+                read(tt + 2, ga, ka, qa, va, ba);
+                token(tt + 1, gb, kb, qb, vb, bb);
+            }
         }
         __syncthreads();
-        for (int idx = tid; idx < count * kScanCols; idx += threads) {
-            const int tt = idx / kScanCols, c = idx % kScanCols;
-            if (col0 + c < dv) {
-                float o = 0.f;
-                for (int w = 0; w < nw; ++w) o += part_s[(tt * nw + w) * kScanCols + c];
-                out[(static_cast<size_t>(t0 + base + tt) * heads + h) * dv + col0 + c] = o;
-            }
+#pragma unroll
+        for (int u = 0; u < VL; ++u) {
+            const int idx = tid + u * THREADS;
+            const int tt = idx / WG_COLS, cc = idx % WG_COLS;
+            if (tt < count && col0 + cc < dv) out[(static_cast<size_t>(t0 + base + tt) * heads + h) * dv + col0 + cc] = o_s[idx];
         }
     }
     if (has_col) {
 #pragma unroll
-        for (int i = 0; i < DKR; ++i) {
-            const int r = wave * DKR + i;
+        for (int i = 0; i < R; ++i) {
+            const int r = sl * R + i;
             if (r < dk) state[static_cast<size_t>(r) * dv + j] = s[i];
         }
     }
+}
+
+template <int SLICES, int R>
+static void launch_delta(const float* ops, int ops_width, int q_off, int k_off, int v_off, int beta_off, const float* decay,
+                         float* states, size_t state_stride, const int32_t* slots, const unsigned char* fresh,
+                         const int32_t* q_start, const int32_t* q_len, int n_seqs, float* out, int heads, int kv_heads, int dk,
+                         int dv, hipStream_t s) {
+    constexpr int cols = kWave / SLICES;
+    dim3 grid(n_seqs, heads, (dv + cols - 1) / cols);
+    delta_rule_scan_kernel<SLICES, R><<<grid, kWave, 0, s>>>(ops, ops_width, q_off, k_off, v_off, beta_off, decay, states,
+                                                            state_stride, slots, fresh, q_start, q_len, out, heads, kv_heads, dk, dv);
 }
 
 }  // namespace egpt
@@ -534,29 +605,42 @@ extern "C" int egpt_delta_rule_scan(const float* ops, int ops_width, int q_off, 
     if (q_off + kv_heads * dk > ops_width || k_off + kv_heads * dk > ops_width || v_off + heads * dv > ops_width ||
         beta_off + heads > ops_width || state_stride < static_cast<long long>(heads) * dk * dv)
         return EGPT_BAD_ARGUMENT;
-    if (dk > 1024 || heads > 65535 || (dv + kScanCols - 1) / kScanCols > 65535) return EGPT_UNSUPPORTED_SIZE;
+    if (dk > 1024 || heads > 65535 || dv > 65535) return EGPT_UNSUPPORTED_SIZE;
     if (n_tokens == 0) return EGPT_OK;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    // rows of the state per wavefront, and wavefronts per workgroup (at most 16)
-    const int dkr = dk <= 256 ? 16 : (dk <= 512 ? 32 : 64);
-    const int nw = (dk + dkr - 1) / dkr, dkp = nw * dkr;
-    // as many tokens to a batch as fit 60 KB of LDS beside the two buffers in which the wavefronts' sums meet
-    const size_t per_token = (3 * static_cast<size_t>(dkp) + kScanCols + static_cast<size_t>(nw) * kScanCols) * sizeof(float) + 4;
-    const size_t fixed = (2 * static_cast<size_t>(nw) * kScanCols + 4) * sizeof(float);
-    int tb = static_cast<int>((60 * 1024 - fixed) / per_token);
-    tb = tb > 32 ? 32 : (tb < 1 ? 1 : tb);
-    const size_t lds = fixed + per_token * tb + 16;
-    dim3 grid(n_seqs, heads, (dv + kScanCols - 1) / kScanCols);
+    // A lane keeps 4, 8 or 16 key channels of a column: the fewest that ask for no more than 1,024 wavefronts (a prompt of
+    // one request walks its tokens on as many wavefronts as the state has columns times slices, and a wavefront's time per
+    // token is its instructions per token: fewer rows, more wavefronts, a shorter walk; a step of many requests fills the
+    // GPU with 16 rows to a lane); as many slices of the key channels as cover dk, a power of two.
+    int rows = 16, slices = 1;
+    for (int r = 4; r <= 16; r *= 2) {
+        int sl = 1;
+        while (sl * r < dk) sl <<= 1;
+        if (sl > 64) continue;
+        const long long wavefronts = static_cast<long long>(n_seqs) * heads * ((dv + 64 / sl - 1) / (64 / sl));
+        if (wavefronts <= 1024 || r == 16) {
+            rows = r, slices = sl;
+            break;
+        }
+    }
     const size_t stride = static_cast<size_t>(state_stride);
-    if (dkr == 16)
-        delta_rule_scan_kernel<16><<<grid, nw * kWave, lds, s>>>(ops, ops_width, q_off, k_off, v_off, beta_off, decay, states, stride,
-                                                                 slots, fresh, q_start, q_len, out, heads, kv_heads, dk, dv, tb);
-    else if (dkr == 32)
-        delta_rule_scan_kernel<32><<<grid, nw * kWave, lds, s>>>(ops, ops_width, q_off, k_off, v_off, beta_off, decay, states, stride,
-                                                                 slots, fresh, q_start, q_len, out, heads, kv_heads, dk, dv, tb);
-    else
-        delta_rule_scan_kernel<64><<<grid, nw * kWave, lds, s>>>(ops, ops_width, q_off, k_off, v_off, beta_off, decay, states, stride,
-                                                                 slots, fresh, q_start, q_len, out, heads, kv_heads, dk, dv, tb);
+#define EGPT_DELTA(S)                                                                                                              \
+    case S:                                                                                                                        \
+        if (rows == 4)                                                                                                             \
+            launch_delta<S, 4>(ops, ops_width, q_off, k_off, v_off, beta_off, decay, states, stride, slots, fresh, q_start, q_len, \
+                               n_seqs, out, heads, kv_heads, dk, dv, s);                                                           \
+        else if (rows == 8)                                                                                                        \
+            launch_delta<S, 8>(ops, ops_width, q_off, k_off, v_off, beta_off, decay, states, stride, slots, fresh, q_start, q_len, \
+                               n_seqs, out, heads, kv_heads, dk, dv, s);                                                           \
+        else                                                                                                                       \
+            launch_delta<S, 16>(ops, ops_width, q_off, k_off, v_off, beta_off, decay, states, stride, slots, fresh, q_start, q_len, \
+                                n_seqs, out, heads, kv_heads, dk, dv, s);                                                          \
+        break;
+    switch (slices) {
+        EGPT_DELTA(1) EGPT_DELTA(2) EGPT_DELTA(4) EGPT_DELTA(8) EGPT_DELTA(16) EGPT_DELTA(32) EGPT_DELTA(64)
+        default: return EGPT_UNSUPPORTED_SIZE;
+    }
+#undef EGPT_DELTA
     EGPT_CHECK_LAUNCH();
     return EGPT_OK;
 }
