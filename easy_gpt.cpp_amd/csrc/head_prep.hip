@@ -343,6 +343,47 @@ __global__ __launch_bounds__(kWave) void head_norm_gate_kernel(ProductView<float
     }
 }
 
+// The same for heads of many values: a workgroup of four wavefronts per (token, head), the statistics through LDS.
+template <typename T>
+__global__ __launch_bounds__(256) void head_norm_gate_wide_kernel(ProductView<float> x, ProductView<T> xa, int x_width,
+                                                                    const T* __restrict__ weight, float eps, ProductView<T> g,
+                                                                    int gate_width, int gate_off, int gate_act, T* __restrict__ out,
+                                                                    int heads, int dv) {
+    __shared__ float scratch[16];
+    const int t = blockIdx.x, h = blockIdx.y;
+    const size_t xr = static_cast<size_t>(t) * x_width + static_cast<size_t>(h) * dv;
+    const bool act_typed = xa.present();
+    constexpr int kKeep = 8;                              // values of the head that a thread keeps between the two passes
+    float v[kKeep];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < kKeep; ++i) {
+        const int d = threadIdx.x + i * 256;
+        v[i] = d < dv ? (act_typed ? xa.at(xr + d) : x.at(xr + d)) : 0.f;
+        ss = fmaf(v[i], v[i], ss);
+    }
+    for (int d = threadIdx.x + kKeep * 256; d < dv; d += 256) {
+        const float u = act_typed ? xa.at(xr + d) : x.at(xr + d);
+        ss = fmaf(u, u, ss);
+    }
+    const float inv = inv_rms(block_sum(ss, scratch), 1.0f / static_cast<float>(dv), eps);
+    auto put = [&](int d, float value) {
+        float y = value * inv * to_float(weight[d]);
+        if (g.present()) {
+            const float gate = g.at(static_cast<size_t>(t) * gate_width + gate_off + h * dv + d);
+            const float sig = 1.0f / (1.0f + expf(-gate));
+            y *= gate_act == 0 ? gate * sig : (gate_act == 1 ? sig : gate);
+        }
+        out[(static_cast<size_t>(t) * heads + h) * dv + d] = from_float<T>(y);
+    };
+#pragma unroll
+    for (int i = 0; i < kKeep; ++i) {
+        const int d = threadIdx.x + i * 256;
+        if (d < dv) put(d, v[i]);
+    }
+    for (int d = threadIdx.x + kKeep * 256; d < dv; d += 256) put(d, act_typed ? xa.at(xr + d) : x.at(xr + d));
+}
+
 template <typename T>
 static ProductView<T> view_of(const void* p, int n_splits, size_t split_stride) {
     ProductView<T> v;
@@ -519,6 +560,20 @@ extern "C" int egpt_head_norm_gate(const void* x, int x_splits, int x_is_act, in
     xv.partial = x_splits > 0 ? static_cast<const float*>(x) : nullptr;
     xv.n_splits = x_splits;
     xv.split_stride = static_cast<size_t>(n_tokens) * x_width;
+    if (dv > 256) {                                       // heads of many values: four wavefronts a head
+        if (dtype == 0)
+            head_norm_gate_wide_kernel<float><<<grid, 256, 0, s>>>(xv, view_of<float>(x_is_act ? x : nullptr, 0, 0), x_width,
+                                                                   static_cast<const float*>(weight), eps,
+                                                                   view_of<float>(gate, gate_splits, stride), gate_width, gate_off,
+                                                                   gate_act, static_cast<float*>(out), heads, dv);
+        else
+            head_norm_gate_wide_kernel<bf16_t><<<grid, 256, 0, s>>>(xv, view_of<bf16_t>(x_is_act ? x : nullptr, 0, 0), x_width,
+                                                                    static_cast<const bf16_t*>(weight), eps,
+                                                                    view_of<bf16_t>(gate, gate_splits, stride), gate_width, gate_off,
+                                                                    gate_act, static_cast<bf16_t*>(out), heads, dv);
+        EGPT_CHECK_LAUNCH();
+        return EGPT_OK;
+    }
     if (dtype == 0)
         head_norm_gate_kernel<float><<<grid, kWave, 0, s>>>(xv, view_of<float>(x_is_act ? x : nullptr, 0, 0), x_width,
                                                             static_cast<const float*>(weight), eps,

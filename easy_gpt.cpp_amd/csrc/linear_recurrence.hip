@@ -291,49 +291,52 @@ constexpr int kMaxTaps = 16;
 // channels are then made unit vectors head by head, y / sqrt(sum y^2 + unit_eps), the first scaled_heads of them also
 // times `scale`.  Behind the channels the output row holds the sigmoid of the n_sig columns from sig_off on.  All float32.
 template <typename T>
-__global__ __launch_bounds__(256) void short_conv_kernel(
+__global__ __launch_bounds__(1024) void short_conv_kernel(
     ProductView<T> proj, int proj_width, int col0, const T* __restrict__ conv_w, int taps, int channels, int unit_heads,
     int unit_dim, int scaled_heads, float scale, float unit_eps, int sig_off, int n_sig, const float* __restrict__ states,
     size_t state_stride, const int32_t* __restrict__ slots, const unsigned char* __restrict__ fresh,
     const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len, float* __restrict__ out, int out_width) {
     extern __shared__ float conv_s[];
-    const int b = blockIdx.x, i = blockIdx.y;
-    if (i >= q_len[b]) return;
+    const int b = blockIdx.x;
+    const int n = q_len[b];
     const int t0 = q_start[b];
-    const size_t t = static_cast<size_t>(t0 + i);
     const float* hist = states + static_cast<size_t>(slots[b]) * state_stride;
     const bool anew = fresh != nullptr && fresh[b] != 0;
-    for (int c = threadIdx.x; c < channels; c += blockDim.x) {
-        float acc = 0.f;
-        for (int j = 0; j < taps; ++j) {
-            const int src = i - (taps - 1) + j;
-            float x;
-            if (src >= 0)
-                x = proj.at(static_cast<size_t>(t0 + src) * proj_width + col0 + c);
-            else
-                x = anew ? 0.f : hist[static_cast<size_t>(src + taps - 1) * channels + c];
-            acc = fmaf(x, to_float(conv_w[static_cast<size_t>(c) * taps + j]), acc);
-        }
-        conv_s[c] = acc / (1.0f + expf(-acc));
-    }
-    __syncthreads();
-    float* orow = out + t * out_width;
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave, n_waves = blockDim.x / kWave;
-    for (int hh = wave; hh < unit_heads; hh += n_waves) {
-        const float* head = conv_s + hh * unit_dim;
-        float ss = 0.f;
-        for (int d = lane; d < unit_dim; d += kWave) ss = fmaf(head[d], head[d], ss);
-        float f = 1.0f / sqrtf(wave_sum(ss) + unit_eps);
-        if (hh < scaled_heads) f *= scale;
-        for (int d = lane; d < unit_dim; d += kWave) orow[hh * unit_dim + d] = head[d] * f;
+    for (int i = blockIdx.y; i < n; i += gridDim.y) {                   // (the grid has a workgroup per token of the longest portion, up to 65,535)
+        const size_t t = static_cast<size_t>(t0 + i);
+        __syncthreads();                                                 // the token before is written out
+        for (int c = threadIdx.x; c < channels; c += blockDim.x) {
+            float acc = 0.f;
+            for (int j = 0; j < taps; ++j) {
+                const int src = i - (taps - 1) + j;
+                float x;
+                if (src >= 0)
+                    x = proj.at(static_cast<size_t>(t0 + src) * proj_width + col0 + c);
+                else
+                    x = anew ? 0.f : hist[static_cast<size_t>(src + taps - 1) * channels + c];
+                acc = fmaf(x, to_float(conv_w[static_cast<size_t>(c) * taps + j]), acc);
+            }
+            conv_s[c] = acc / (1.0f + expf(-acc));
+        }
+        __syncthreads();
+        float* orow = out + t * out_width;
+        for (int hh = wave; hh < unit_heads; hh += n_waves) {
+            const float* head = conv_s + hh * unit_dim;
+            float ss = 0.f;
+            for (int d = lane; d < unit_dim; d += kWave) ss = fmaf(head[d], head[d], ss);
+            float f = 1.0f / sqrtf(wave_sum(ss) + unit_eps);
+            if (hh < scaled_heads) f *= scale;
+            for (int d = lane; d < unit_dim; d += kWave) orow[hh * unit_dim + d] = head[d] * f;
+        }
+        for (int c = unit_heads * unit_dim + threadIdx.x; c < channels; c += blockDim.x) orow[c] = conv_s[c];
+        for (int c = threadIdx.x; c < n_sig; c += blockDim.x)
+            orow[channels + c] = 1.0f / (1.0f + expf(-proj.at(t * proj_width + sig_off + c)));
     }
-    for (int c = unit_heads * unit_dim + threadIdx.x; c < channels; c += blockDim.x) orow[c] = conv_s[c];
-    for (int c = threadIdx.x; c < n_sig; c += blockDim.x)
-        orow[channels + c] = 1.0f / (1.0f + expf(-proj.at(t * proj_width + sig_off + c)));
 }
 
 // After a step: a request's record takes the last taps - 1 inputs of its convolutions (those of this step, and, where the
-// step brought fewer, what the record held, moved up).  One workgroup per request; a thread owns a channel's column.
+// step brought fewer, what the record held, moved up).  Workgroups per request and 256 channels; a thread owns a channel's column.
 template <typename T>
 __global__ __launch_bounds__(256) void conv_carry_kernel(ProductView<T> proj, int proj_width, int col0, int taps, int channels,
                                                          float* __restrict__ states, size_t state_stride,
@@ -345,7 +348,7 @@ __global__ __launch_bounds__(256) void conv_carry_kernel(ProductView<T> proj, in
     const int t0 = q_start[b];
     float* hist = states + static_cast<size_t>(slots[b]) * state_stride;
     const bool anew = fresh != nullptr && fresh[b] != 0;
-    for (int c = threadIdx.x; c < channels; c += blockDim.x) {
+    for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < channels; c += gridDim.y * blockDim.x) {
         float keep[kMaxTaps];
 #pragma unroll
         for (int j = 0; j < kMaxTaps; ++j) {
@@ -565,28 +568,31 @@ extern "C" int egpt_short_conv(const void* proj, int n_splits, int proj_width, i
     if (static_cast<long long>(unit_heads) * unit_dim > channels || col0 + channels > proj_width ||
         (n_sig > 0 && (sig_off < 0 || sig_off + n_sig > proj_width)) || state_stride < static_cast<long long>(taps - 1) * channels)
         return EGPT_BAD_ARGUMENT;
-    if (taps > kMaxTaps || channels > 15360 || max_q_len > 65535) return EGPT_UNSUPPORTED_SIZE;     // a token's channels lie in LDS
+    if (taps > kMaxTaps || channels > 15360) return EGPT_UNSUPPORTED_SIZE;     // a token's channels lie in LDS
     if (n_tokens == 0 || max_q_len == 0) return EGPT_OK;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const size_t stride = static_cast<size_t>(n_tokens) * proj_width;
     const size_t lds = static_cast<size_t>(channels) * sizeof(float);
     const int out_width = channels + n_sig;
-    dim3 grid(n_seqs, max_q_len);
+    dim3 grid(n_seqs, max_q_len > 65535 ? 65535 : max_q_len);
+    dim3 carry_grid(n_seqs, (channels + 255) / 256);
+    // (a token's channels are walked in rounds of the workgroup's width: wide workgroups where the channels are many)
+    const int width = channels > 512 ? 1024 : 256;
     if (dtype == 0) {
-        short_conv_kernel<float><<<grid, 256, lds, s>>>(scan_view<float>(proj, n_splits, stride), proj_width, col0,
+        short_conv_kernel<float><<<grid, width, lds, s>>>(scan_view<float>(proj, n_splits, stride), proj_width, col0,
                                                         static_cast<const float*>(conv_w), taps, channels, unit_heads, unit_dim,
                                                         scaled_heads, scale, unit_eps, sig_off, n_sig, states,
                                                         static_cast<size_t>(state_stride), slots, fresh, q_start, q_len, out, out_width);
         if (taps > 1)
-            conv_carry_kernel<float><<<n_seqs, 256, 0, s>>>(scan_view<float>(proj, n_splits, stride), proj_width, col0, taps, channels,
+            conv_carry_kernel<float><<<carry_grid, 256, 0, s>>>(scan_view<float>(proj, n_splits, stride), proj_width, col0, taps, channels,
                                                             states, static_cast<size_t>(state_stride), slots, fresh, q_start, q_len);
     } else {
-        short_conv_kernel<bf16_t><<<grid, 256, lds, s>>>(scan_view<bf16_t>(proj, n_splits, stride), proj_width, col0,
+        short_conv_kernel<bf16_t><<<grid, width, lds, s>>>(scan_view<bf16_t>(proj, n_splits, stride), proj_width, col0,
                                                          static_cast<const bf16_t*>(conv_w), taps, channels, unit_heads, unit_dim,
                                                          scaled_heads, scale, unit_eps, sig_off, n_sig, states,
                                                          static_cast<size_t>(state_stride), slots, fresh, q_start, q_len, out, out_width);
         if (taps > 1)
-            conv_carry_kernel<bf16_t><<<n_seqs, 256, 0, s>>>(scan_view<bf16_t>(proj, n_splits, stride), proj_width, col0, taps, channels,
+            conv_carry_kernel<bf16_t><<<carry_grid, 256, 0, s>>>(scan_view<bf16_t>(proj, n_splits, stride), proj_width, col0, taps, channels,
                                                              states, static_cast<size_t>(state_stride), slots, fresh, q_start, q_len);
     }
     EGPT_CHECK_LAUNCH();

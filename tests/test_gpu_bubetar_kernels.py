@@ -119,7 +119,7 @@ def test_latent_preparation_takes_queries_from_a_product_of_their_own(k, dtype, 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("heads, dv, x_extra, x_splits, act", [(1, 48, 0, 3, "sigmoid"), (4, 12, 0, 1, "factor"), (1, 24, 40, 2, None),
-                                                              (1, 10, 19, -1, None), (3, 70, 0, 0, "silu"), (1, 1300, 0, 1, "sigmoid")])
+                                                              (1, 10, 19, -1, None), (3, 70, 0, 0, "silu"), (1, 1300, 0, 1, "sigmoid"), (2, 2500, 7, 2, "factor"), (1, 257, 0, 0, None)])
 def test_heads_are_normed_from_the_first_columns_of_a_row_and_gated(k, dtype, heads, dv, x_extra, x_splits, act):
     t, eps = 6, 1e-5
     width = heads * dv + x_extra
