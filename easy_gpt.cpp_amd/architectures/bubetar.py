@@ -67,8 +67,9 @@ def _mixer_spec(layer: BubetarLayer, p: str, eps: float) -> PartSpec:
             dict(n_heads=right.heads, n_kv_heads=right.kv_heads, key_dim=right.dim, value_dim=right.vdim, taps=right.conv,
                  eps=eps, unit_eps=UNIT_EPS),
             prefix=p + "right.")
+    # (the sum of the two sides is left to the norm behind the mixer, which every layer of this design has)
     return PartSpec("side_by_side", dict(left=lspec, right=rspec, eps=eps, join="weighted_sum",
-                                         factors=(m.left_scale, m.right_scale)), prefix=p)
+                                         factors=(m.left_scale, m.right_scale), deferred=True), prefix=p)
 
 
 def _layer_spec(layer: BubetarLayer, index: int, eps: float) -> LayerSpec:

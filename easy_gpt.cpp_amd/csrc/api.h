@@ -201,9 +201,10 @@ int egpt_embed_positions(const int32_t* ids, const int32_t* positions, const voi
 // x = h + mult * LN(y) * post_w (LN without bias; y a product: one tensor or float32 partial sums).  With hist (float32
 // [n_hist + 1][n_rows][hidden]) x is stored as hist[n_hist] and v = sum_(j <= n_hist) mix[j] * hist[j], else v = x.
 // h_out = v (h_out may be h).  With next_w, out = LN(v) * next_w in the activation type.
-int egpt_post_norm_add(const float* h, const void* y, int y_splits, const void* post_w, float eps, float mult, float* hist,
-                       int n_hist, const float* mix, float* h_out, const void* next_w, void* out, int n_rows, int hidden,
-                       int dtype, void* stream);
+// (y2, may be null: a second product; the branch is then fy * y + fy2 * y2)
+int egpt_post_norm_add(const float* h, const void* y, int y_splits, const void* y2, int y2_splits, float fy, float fy2,
+                       const void* post_w, float eps, float mult, float* hist, int n_hist, const float* mix, float* h_out,
+                       const void* next_w, void* out, int n_rows, int hidden, int dtype, void* stream);
 // x = cap * tanh(x / cap) in place.
 // x <- x * scale; then, with cap > 0, x <- cap * tanh(x / cap)
 int egpt_tanh_cap(float* x, float scale, float cap, long long n, void* stream);

@@ -120,12 +120,12 @@ __global__ __launch_bounds__(256) void embed_positions_kernel(const int32_t* __r
 }
 
 // A branch's output joins the stream behind a norm of its own:  x = h + mult * LN(y) * post_w  (LN without bias, the
-// statistics of y's row in two passes over LDS).  With a history (every earlier result of the depth, float32
+// statistics of y's row in two passes over LDS).  With a second product y2 the branch is fy * y + fy2 * y2.  With a history (every earlier result of the depth, float32
 // [n_hist + 1][rows][hidden]) x is kept as result n_hist and what goes on is the weighted sum
 // v = sum_(j <= n_hist) mix[j] * hist[j]; otherwise v = x.  v is written to h_out (which may be h itself), and with a
 // next norm's weight LN(v) * next_w is written to `out` in the activation type.  One workgroup per row.
 template <typename T>
-__global__ __launch_bounds__(256) void post_norm_add_kernel(const float* h, ProductView<T> y,
+__global__ __launch_bounds__(256) void post_norm_add_kernel(const float* h, ProductView<T> y, ProductView<T> y2, float fy, float fy2,
                                                             const T* __restrict__ post_w, float eps, float mult,
                                                             float* hist, int n_hist, size_t hist_stride,
                                                             const float* __restrict__ mix, float* h_out,
@@ -135,8 +135,10 @@ __global__ __launch_bounds__(256) void post_norm_add_kernel(const float* h, Prod
     const size_t base = static_cast<size_t>(blockIdx.x) * hidden;
     const float inv_n = 1.0f / static_cast<float>(hidden);
     float sum = 0.f;
+    const bool two = y2.present();                       // the branch is fy * y + fy2 * y2: two products not yet added up
     for (int j = threadIdx.x; j < hidden; j += blockDim.x) {
-        const float v = y.at(base + j);
+        float v = y.at(base + j);
+        if (two) v = fy * v + fy2 * y2.at(base + j);
         row_s[j] = v;
         sum += v;
     }
@@ -259,10 +261,11 @@ extern "C" int egpt_embed_positions(const int32_t* ids, const int32_t* positions
     return EGPT_OK;
 }
 
-extern "C" int egpt_post_norm_add(const float* h, const void* y, int y_splits, const void* post_w, float eps, float mult,
+extern "C" int egpt_post_norm_add(const float* h, const void* y, int y_splits, const void* y2, int y2_splits, float fy, float fy2,
+                                  const void* post_w, float eps, float mult,
                                   float* hist, int n_hist, const float* mix, float* h_out, const void* next_w, void* out,
                                   int n_rows, int hidden, int dtype, void* stream) {
-    if (!h || !y || !post_w || !h_out || n_rows < 0 || hidden <= 0 || y_splits < 0 || n_hist < 0 || (dtype != 0 && dtype != 1))
+    if (!h || !y || !post_w || !h_out || n_rows < 0 || hidden <= 0 || y_splits < 0 || y2_splits < 0 || n_hist < 0 || (dtype != 0 && dtype != 1))
         return EGPT_BAD_ARGUMENT;
     if ((hist != nullptr) != (mix != nullptr) || (next_w != nullptr) != (out != nullptr)) return EGPT_BAD_ARGUMENT;
     if (hidden > 16384) return EGPT_UNSUPPORTED_SIZE;          // a row lies in LDS
@@ -272,10 +275,12 @@ extern "C" int egpt_post_norm_add(const float* h, const void* y, int y_splits, c
     const size_t lds = static_cast<size_t>(hidden) * sizeof(float);
     if (dtype == 0)
         post_norm_add_kernel<float><<<n_rows, 256, lds, s>>>(h, stream_view<float>(y, y_splits, stride),
+                                                             stream_view<float>(y2, y2 ? y2_splits : 0, stride), fy, fy2,
                                                              static_cast<const float*>(post_w), eps, mult, hist, n_hist, stride, mix,
                                                              h_out, static_cast<const float*>(next_w), static_cast<float*>(out), hidden);
     else
         post_norm_add_kernel<bf16_t><<<n_rows, 256, lds, s>>>(h, stream_view<bf16_t>(y, y_splits, stride),
+                                                              stream_view<bf16_t>(y2, y2 ? y2_splits : 0, stride), fy, fy2,
                                                               static_cast<const bf16_t*>(post_w), eps, mult, hist, n_hist, stride, mix,
                                                               h_out, static_cast<const bf16_t*>(next_w), static_cast<bf16_t*>(out), hidden);
     EGPT_CHECK_LAUNCH();

@@ -65,7 +65,9 @@ Methods of a backend (T tokens, B requests, R rows, act = bfloat16 or float32):
         h += delta; out = (h - mean) / sqrt(mean((h - mean)^2) + eps) * weight + bias; with rows only those, h untouched
   normed_pair_mean(a, b, bias_a|None, bias_b|None, weight_a, weight_b, eps, factor) -> f32[1,T,H]
         factor * (rmsnorm(a + bias_a) * weight_a + rmsnorm(b + bias_b) * weight_b); a, b products (act or partial sums)
-  tanh_cap(x f32[...], cap)                    x = cap * tanh(x / cap) in place
+  tanh_cap(x f32[...], cap, scale=1)           x = cap * tanh(scale * x / cap) in place (cap None: scale * x)
+  post_norm_add(h f32[T,H], y, post_weight act[H], eps, mult, ...)     h += mult * LN(y) * post_weight, LN without bias; y a product
+        (act [T, H] or float32 partial sums) or a ProductSum of two
   whole_norm_store(proj, bias act[W]|None, q_out act[T,nq*dk], q_weight act[nq*dk]|None, k_weight act[nkv*dk]|None, eps,
                    positions i32[T], coef, every, slots, k_cache, v_cache, nq, nkv, dk, dv, page_size)
         proj rows are [nq heads of dk | nkv heads of dk | nkv heads of dv | ...]; the bias is added, queries (all heads at
@@ -93,6 +95,17 @@ from __future__ import annotations
 import contextlib
 
 _backend = None
+
+
+class ProductSum:
+    """factor_a * a + factor_b * b of two products (each act [T, H] or float32 partial sums [S, T, H]) that nothing has
+    added up yet: what two mixers side by side hand to an arrangement whose next kernel (`post_norm_add`) takes it as it
+    is, so that the sum costs no kernel of its own."""
+
+    __slots__ = ("a", "factor_a", "b", "factor_b")
+
+    def __init__(self, a, factor_a, b, factor_b):
+        self.a, self.factor_a, self.b, self.factor_b = a, float(factor_a), b, float(factor_b)
 
 
 class KernelBackend:

@@ -10,7 +10,7 @@ import ctypes
 
 import torch
 
-from . import KernelBackend, KernelsUnavailable
+from . import KernelBackend, KernelsUnavailable, ProductSum
 
 _F32, _BF16, _I32, _I64 = torch.float32, torch.bfloat16, torch.int32, torch.int64
 _DT = {_F32: 0, _BF16: 1}
@@ -28,7 +28,7 @@ def _load_library() -> ctypes.CDLL:
         lib = ctypes.CDLL(path)
     except (build.BuildError, OSError) as e:
         raise KernelsUnavailable(f"the HIP kernel library could not be built or loaded: {e}") from e
-    if lib.egpt_abi_version() != 23:
+    if lib.egpt_abi_version() != 24:
         raise KernelsUnavailable(f"{path} has an unexpected ABI version")
     return lib
 
@@ -109,7 +109,7 @@ class HipKernels(KernelBackend):
             "egpt_window_attention_tiled": [vp, vp, vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, i, f, i, i, vp, vp, i,
                                             i, vp, i, i, i, vp],
             "egpt_embed_positions": [vp, vp, vp, vp, vp, i, i, i, i, i, vp],
-            "egpt_post_norm_add": [vp, vp, i, vp, f, f, vp, i, vp, vp, vp, vp, i, i, i, vp],
+            "egpt_post_norm_add": [vp, vp, i, vp, i, f, f, vp, f, f, vp, i, vp, vp, vp, vp, i, i, i, vp],
             "egpt_bounded_gate": [vp, i, i, i, vp, vp, vp, i, i, i, vp],
             "egpt_ff_activation": [vp, i, i, i, i, vp, f, i, vp, i, i, vp],
             "egpt_moe_up": [vp, vp, vp, vp, vp, i, i, i, i, i, i, vp],
@@ -1106,13 +1106,17 @@ class HipKernels(KernelBackend):
 
     def post_norm_add(self, h, y, post_weight, eps, mult, history=None, n_history=0, mix=None, next_weight=None, h_out=None):
         """x = h + mult * LN(y) * post_weight, LN without bias over y's rows (y a product: act [T, H] or float32 partial
-        sums [S, T, H]).  With history (float32 [n, T, H], n > n_history) x is stored as history[n_history] and what goes on
+        sums [S, T, H]; or a `ProductSum` of two such products, which is added up here with its factors).  With history (float32 [n, T, H], n > n_history) x is stored as history[n_history] and what goes on
         is v = sum_(j <= n_history) mix[j] * history[j] (mix float32 [n_history + 1]); else v = x.  v is written to h_out
         (h itself if None).  Returns LN(v) * next_weight as act [T, H], or None without next_weight."""
         dt = self._act(post_weight, "post_weight")
         t, hidden = h.shape
         self._need(h, "h", _F32)
         self._need(post_weight, "post_weight", None, (hidden,))
+        y2, splits2, fa, fb = None, 0, 1.0, 0.0
+        if isinstance(y, ProductSum):
+            y, y2, fa, fb = y.a, y.b, y.factor_a, y.factor_b
+            splits2 = self._product(y2, "the sum's second product", post_weight.dtype, t, hidden)
         splits = self._product(y, "y", post_weight.dtype, t, hidden)
         if history is not None:
             self._need(history, "history", _F32)
@@ -1125,7 +1129,8 @@ class HipKernels(KernelBackend):
         if next_weight is not None:
             self._need(next_weight, "next_weight", post_weight.dtype, (hidden,))
             out = torch.empty((t, hidden), dtype=post_weight.dtype, device=h.device)
-        self._run("egpt_post_norm_add", h.data_ptr(), y.data_ptr(), splits, post_weight.data_ptr(), float(eps), float(mult),
+        self._run("egpt_post_norm_add", h.data_ptr(), y.data_ptr(), splits, self._ptr(y2), splits2, float(fa), float(fb),
+                  post_weight.data_ptr(), float(eps), float(mult),
                   self._ptr(history), int(n_history), self._ptr(mix) if history is not None else None, h_out.data_ptr(),
                   self._ptr(next_weight), self._ptr(out), t, hidden, dt, self._stream())
         return out

@@ -198,10 +198,12 @@ class GatedLinearAttention(_Branch):
 
 class SideBySide(Mixer):
     def __init__(self, prefix: str, hidden_size: int, left: PartSpec, right: PartSpec, eps: float, factor: float = 0.5,
-                 names: dict | None = None, join: str = "normed_mean", factors: tuple | None = None):
+                 names: dict | None = None, join: str = "normed_mean", factors: tuple | None = None, deferred: bool = False):
         """left, right: the two branches (mixers that offer `branch`).  join 'normed_mean': each output is RMS-normed
         over the width with a weight of its own (names: those weights behind `prefix`) and the result is `factor` times
-        their sum; join 'weighted_sum': the result is factors[0] * left + factors[1] * right, no norms, no weights."""
+        their sum; join 'weighted_sum': the result is factors[0] * left + factors[1] * right, no norms, no weights;
+        with `deferred` it is handed on as a `kernels.ProductSum` for an arrangement whose next kernel adds it up (the
+        sandwich arrangement's norm behind the mixer)."""
         if join not in ("normed_mean", "weighted_sum"):
             raise ValueError(f"unknown join '{join}' of two mixers side by side (normed_mean, weighted_sum)")
         if join == "weighted_sum" and (factors is None or len(factors) != 2):
@@ -209,6 +211,7 @@ class SideBySide(Mixer):
         self.prefix, self.hidden_size = prefix, int(hidden_size)
         self.eps, self.factor, self.join = float(eps), float(factor), join
         self.factors = (float(factors[0]), float(factors[1])) if join == "weighted_sum" else None
+        self.deferred = bool(deferred) and join == "weighted_sum"
         self.branches = [make_part("mixer", left, hidden_size=hidden_size), make_part("mixer", right, hidden_size=hidden_size)]
         for b in self.branches:
             if not hasattr(b, "branch"):
@@ -244,6 +247,8 @@ class SideBySide(Mixer):
         outs = [b.branch(x, ctx, cache if b.cache_need() is not None else None, state if b.state_need() is not None else None)
                 for b in self.branches]
         (a, bias_a), (b, bias_b) = outs
+        if self.deferred and bias_a is None and bias_b is None:
+            return kernels.ProductSum(a, self.factors[0], b, self.factors[1])
         if self.join == "weighted_sum":
             return kernels.backend().normed_pair_mean(a, b, bias_a, bias_b, None, None, self.eps, self.factors[0],
                                                       factor_b=self.factors[1], act_dtype=x.dtype)

@@ -422,6 +422,10 @@ class EmulatedKernels(KernelBackend):
             mu = x.mean(-1, keepdim=True)
             return (x - mu) / torch.sqrt(((x - mu) ** 2).mean(-1, keepdim=True) + eps) * w.to(F64)
 
+        from easy_gpt.cpp_amd.kernels import ProductSum
+
+        if isinstance(y, ProductSum):
+            y = y.factor_a * _whole(y.a).to(F64) + y.factor_b * _whole(y.b).to(F64)
         x = h.to(F64) + mult * normed(_whole(y).to(F64), post_weight)
         if history is not None:
             history[n_history].copy_(x.to(history.dtype))

@@ -155,6 +155,23 @@ def test_two_branches_are_added_with_a_factor_each(k, dtype, hidden, sa, sb):
     close(out[0], 0.6 * a + 1.1 * b, torch.float32, "weighted sum of two branches")
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("hidden, sa, sb", [(48, 3, 1), (256, 0, 2), (1000, 2, 0)])
+def test_the_norm_behind_a_mixer_adds_up_two_sides_not_yet_joined(k, dtype, hidden, sa, sb):
+    from easy_gpt.cpp_amd.kernels import ProductSum
+
+    t, eps = 6, 1e-5
+    h = rnd(t, hidden, seed=40, scale=2.0)
+    a_given, a = product(rnd(t, hidden, seed=41, scale=2.0) + 0.3, dtype, sa)
+    b_given, b = product(rnd(t, hidden, seed=42, scale=0.7), dtype, sb)
+    post, nxt = rnd(hidden, seed=43, dtype=dtype) + 1, rnd(hidden, seed=44, dtype=dtype) + 1
+    x = h.to(F64) + P.layer_norm(0.6 * a - 1.1 * b, post.to(F64), eps)
+    h_dev = h.to(DEV).clone()
+    got = k.post_norm_add(h_dev, ProductSum(a_given, 0.6, b_given, -1.1), post.to(DEV), eps, 1.0, next_weight=nxt.to(DEV))
+    close(h_dev, x, torch.float32, "the stream")
+    close(got, P.layer_norm(x, nxt.to(F64), eps), dtype, "the next norm")
+
+
 def test_logits_take_a_factor_and_a_cap(k):
     x = rnd(7, 301, seed=12, scale=9.0)
     y = x.to(DEV).clone()
