@@ -54,7 +54,7 @@ class Rotation:
 
 def _heads(r: KeyReader, where: str, grouped: bool) -> tuple[int, int]:
     heads = r.integer("heads", minimum=1)
-    kv_heads = r.integer("kv_heads", minimum=1) if grouped else heads
+    kv_heads = r.integer("kv_heads", heads, minimum=1) if grouped else heads       # (absent: a key/value head per head)
     if heads % kv_heads:
         raise ConfigError(f"{where}: 'heads' ({heads}) must be a multiple of 'kv_heads' ({kv_heads})")
     return heads, kv_heads
