@@ -461,12 +461,12 @@ def bubetar_config(width, heads, kv_heads, hd, s_heads, s_dim, s_vdim, inner, ra
     delta = {"type": "parallel_2", "mlp": ff,
              "mixer": {"left": {"heads": heads, "kv_heads": kv_heads, "dim": hd, "vdim": hd, "scale": hd ** -0.5,
                                 "mask": {"size": window},
-                                "rot": {"base": 1000000.0, "dims": hd, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}},
+                                "rot": {"base": 500000.0, "dims": hd, "scaling": {"factor": 16.0, "low": 1.0, "high": 8.0, "original": 8192}}},
                        "right": {"heads": s_heads, "kv_heads": s_heads, "dim": s_dim, "vdim": s_vdim, "conv": 4},
                        "left_scale": 1.0, "right_scale": 1.0}}
     layers = [delta, latent, gated, latent]
     assert len(layers) == DESIGN_LAYERS
-    return {"architecture": "Bubetar", "vocab": DESIGN_VOCAB, "width": width, "norm": {"eps": 1e-6}, "logit_scale": 0.5,
+    return {"architecture": "Bubetar", "vocab": DESIGN_VOCAB, "width": width, "norm": {"eps": 1e-6}, "logit_scale": 0.75,
             "logit_softcap": 30.0, "layers": layers}
 
 

@@ -81,27 +81,27 @@ CONFIG_B = config(257, 100, 1e-5, [
     layer(latent(4, 6, 0, 10, 12, 14, 0.45, 10000.0), 40),
     layer(pair_2(softmax_side(2, 2, 14, 14, 0.3, rotation(30000.0, 10), 700), delta_rule(1, 1, 36, 8, 2), 0.9, 1.1), None),
 ])
-# multiples of 16, so that the matrix-core attention runs: heads of 64 and 32, windows of 40 (no multiple of a page or
+# multiples of 16, so that the matrix-core attention runs: heads of 64 and 32, windows of 44 (no multiple of a page or
 # of a chunk of keys) and of 64 (a page's and a chunk's edge), latents of 64 + 32 and 48 + 16, states of 64 x 80 and
 # 160 x 64
 CONFIG_C = config(411, 128, 1e-6, [
-    layer(latent(4, 32, 32, 48, 64, 64, 0.12, 250000.0, dims=16), 192),
-    layer(pair_2(softmax_side(8, 2, 64, 64, 0.1, rotation(500000.0, 32, (8.0, 1.0, 4.0, 256)), 40), delta_rule(4, 2, 64, 80, 4), 0.6, 1.1), 160),
+    layer(latent(4, 32, 32, 48, 64, 64, 0.12, 300000.0, dims=16), 192),
+    layer(pair_2(softmax_side(8, 2, 64, 64, 0.1, rotation(500000.0, 32, (6.0, 1.0, 3.0, 256)), 44), delta_rule(4, 2, 64, 80, 5), 0.65, 1.15), 160),
     layer(pair(softmax_side(4, 4, 32, 64, 0.18, rotation(10000.0, 32)), constant_decay(2, 64, 48, (0.6, 0.995)), 1.2, 0.9), 64),
     layer(pair_2(softmax_side(4, 1, 32, 32, 0.15, rotation(10000.0, 16), 64), delta_rule(1, 1, 160, 64, 2), 1.0, 0.7), 96),
     layer(latent(2, 64, 16, 32, 32, 48, 0.11, 1000.0), None),
-], logit_scale=0.5, logit_softcap=20.0)
+], logit_scale=0.4, logit_softcap=20.0)
 # recurrent pairs alone, each kind twice with sizes of its own; then a model of latent attention alone (no state:
 # every step may replay from a graph)
 CONFIG_D = config(199, 96, 1e-5, [
-    layer(pair(softmax_side(6, 3, 16, 16, 0.3, rotation(10000.0, 16)), constant_decay(3, 8, 40, (0.5, 0.9, 0.999)), 0.8, 1.0), 80),
+    layer(pair(softmax_side(6, 3, 16, 16, 0.3, rotation(10000.0, 16)), constant_decay(3, 8, 40, (0.5, 0.9, 0.998)), 0.8, 1.0), 80),
     layer(pair_2(softmax_side(2, 2, 48, 48, 0.15, rotation(10000.0, 24, (16.0, 1.0, 2.0, 128)), 33), delta_rule(6, 3, 16, 8, 4), 1.0, 1.0), 64),
     layer(pair(softmax_side(2, 1, 24, 8, 0.2, rotation(300.0, 2)), constant_decay(4, 16, 16, (0.7, 0.8, 0.9, 0.95)), 1.1, 0.6), None),
 ], logit_softcap=30.0)
 CONFIG_F = config(150, 72, 1e-5, [
     layer(latent(2, 8, 8, 8, 12, 16, 0.3, 10000.0), 40),
     layer(latent(3, 24, 4, 40, 20, 12, 0.2, 64.0, dims=2), None),
-    layer(latent(6, 4, 12, 4, 8, 40, 0.35, 1e6), 56),
+    layer(latent(6, 4, 12, 4, 8, 40, 0.35, 2e6), 56),
 ], logit_scale=2.0)
 CONFIGS = {"A": (CONFIG_A, 5), "B": (CONFIG_B, 6), "C": (CONFIG_C, 7), "D": (CONFIG_D, 8), "F": (CONFIG_F, 10)}
 # how peaked the attention is drawn (a factor on the queries' norm weights).  Configuration B is six layers deep, has a

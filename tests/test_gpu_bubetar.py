@@ -41,9 +41,9 @@ def match(rows, ref, dtype, what):
 # states of 128 x 128 and two value heads per key head, a constant-decay state of 64 x 128, a window of 96
 CONFIG_E = BM.config(523, 256, 1e-6, [
     BM.layer(BM.latent(4, 64, 64, 64, 96, 256, 0.09, 10000.0), 512),
-    BM.layer(BM.pair_2(BM.softmax_side(4, 2, 128, 128, 0.08, BM.rotation(1e6, 64, (8.0, 1.0, 4.0, 512)), 96), BM.delta_rule(2, 1, 128, 128, 4), 0.6, 1.1), 256),
-    BM.layer(BM.pair(BM.softmax_side(4, 1, 64, 128, 0.12, BM.rotation(10000.0, 32)), BM.constant_decay(2, 64, 128, (0.9, 0.999)), 1.2, 1.1), 384),
-], logit_scale=0.5, logit_softcap=15.0)
+    BM.layer(BM.pair_2(BM.softmax_side(4, 2, 128, 128, 0.08, BM.rotation(5e5, 64, (16.0, 1.0, 8.0, 512)), 96), BM.delta_rule(2, 1, 128, 128, 3), 0.7, 1.2), 256),
+    BM.layer(BM.pair(BM.softmax_side(4, 1, 64, 128, 0.12, BM.rotation(10000.0, 32)), BM.constant_decay(2, 64, 128, (0.9, 0.998)), 1.2, 1.05), 384),
+], logit_scale=0.8, logit_softcap=25.0)
 ALL = dict(BM.CONFIGS, E=(CONFIG_E, 9))
 
 
@@ -110,7 +110,7 @@ def test_mixed_batches_with_pages_and_state_slots_used_again(models, dtype, use_
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["A", "C", "E"])
 def test_long_decoding_passes_every_window_and_carries_the_states(models, name, dtype):
-    """Three tokens as a prompt, then 337 one by one: windows of 12, 40, 64 and 96 tokens pass over decoded tokens alone,
+    """Three tokens as a prompt, then 337 one by one: windows of 12, 44, 64 and 96 tokens pass over decoded tokens alone,
     and the matrices and the convolutions' inputs are carried through all of them."""
     cfg = ALL[name][0]
     reqs = H.make_requests(cfg["vocab"], [340], seed=44)

@@ -29,14 +29,14 @@ def draw_config(seed: int) -> dict:
         dims = r.choice([0, even(2, dim), even(2, dim), dim - dim % 2])
         scaling = None
         if dims and r.random() < 0.6:
-            scaling = (r.choice([2.0, 8.0, 32.0]), 1.0, r.choice([2.0, 4.0]), r.choice([16, 64, 256, 2048]))
-        return BM.rotation(r.choice([50.0, 10000.0, 1e6]), dims, scaling)
+            scaling = (r.choice([2.0, 6.0, 32.0]), 1.0, r.choice([2.0, 3.0]), r.choice([16, 64, 256, 4096]))
+        return BM.rotation(r.choice([50.0, 10000.0, 2e6]), dims, scaling)
 
     def latent():
         dim, rot_dim = size(8, 96), even(0, 64) if not round16 else 16 * r.randint(0, 4)
         dims = 0 if rot_dim == 0 else r.choice([rot_dim, even(2, rot_dim)])
         return BM.latent(r.randint(1, 6), dim, rot_dim, size(8, 96), r.randint(4, 100), size(16, 160), (dim + rot_dim) ** -0.5 * r.choice([1.0, 1.7]),
-                         r.choice([100.0, 10000.0, 250000.0]), dims=dims)
+                         r.choice([100.0, 10000.0, 300000.0]), dims=dims)
 
     def left(window, own_values):
         hq, hk = heads()
