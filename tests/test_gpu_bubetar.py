@@ -184,6 +184,70 @@ def test_a_loud_key_is_seen_to_the_windows_last_position_and_not_beyond(tmp_path
         H.assert_rows_match(H.replay(eng, trace), {"r0": want}, TOL[dtype], f"window {window} {dtype} {what}")
 
 
+def _one_loud_latent(cfg):
+    """Weights of a one-layer model of latent attention in which token 7 leaves a latent that the queries of token 9
+    weigh far above all others: channel 0 of the embedding marks token 7 and is all that the first row of the key/value
+    latent reads, channel 1 marks token 9 and is all that the first row of the queries' latent reads; the first column of
+    the queries' and of the keys' up projections carries both into the first unrotated place of every head."""
+
+    def change(w):
+        m = cfg["layers"][0]["mixer"]
+        g = torch.Generator().manual_seed(2)
+        w["embed"][:] = 0.3 * torch.randn(w["embed"].shape, generator=g)
+        w["embed"][:, :2] = 0.0
+        w["embed"][7, :] = 0.0
+        w["embed"][7, 0] = 6.0
+        w["embed"][9, :] = 0.0
+        w["embed"][9, 1] = 6.0
+        w["l0.norm1"][:] = 1.0
+        width = w["embed"].shape[1]
+        for name, channel, norm in (("dkv", 0, "dkv.norm"), ("dq", 1, "dq.norm")):
+            proj = w[f"l0.mix.{name}"]
+            proj[:] = torch.randn(proj.shape, generator=g) / width ** 0.5
+            proj[:, :2] = 0.0
+            proj[0, :] = 0.0
+            proj[0, channel] = 1.0
+            w[f"l0.mix.{norm}"][:] = 1.0
+        for name, rank in (("uq", m["q_rank"]), ("uk", m["kv_rank"])):
+            up = w[f"l0.mix.{name}"]
+            up[:] = 0.5 * torch.randn(up.shape, generator=g) / rank ** 0.5
+            up[:, 0] = 0.0
+        per_q = m["dim"] + m["rot_dim"]
+        for head in range(m["heads"]):
+            w["l0.mix.uq"][head * per_q, 0] = 1.0
+            w["l0.mix.uk"][head * m["dim"], 0] = 1.0
+        for name in w:
+            w[name] = w[name].to(torch.bfloat16).to(torch.float32)
+
+    return change
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_far_key_among_hundreds_reaches_a_latent_layers_queries(tmp_path, dtype):
+    """One latent stands out at position 3 of 700.  Asking tokens at positions 650 to 699, as a whole prompt, in portions
+    and decoded one by one, against the plain implementation, which also shows that the rows differ by far more than the
+    tolerance from those of the same prompt without that token (so a far key that is lost cannot pass)."""
+    cfg = BM.config(64, 48, 1e-5, [BM.layer(BM.latent(3, 12, 8, 20, 10, 14, 1.0, 10000.0), None)])
+    path = BM.write_model(str(tmp_path / "m"), cfg, 4, change=_one_loud_latent(cfg))
+    g = torch.Generator().manual_seed(5)
+    n = 700
+    tokens = torch.randint(10, 64, (n,), generator=g).tolist()
+    tokens[3] = 7
+    asks = [650, 677, 698, 699]
+    for p in asks:
+        tokens[p] = 9
+    c, w = P.read_model(path)
+    want = P.forward(c, w, tokens)
+    without = P.forward(c, w, tokens[:3] + [11] + tokens[4:])
+    for p in asks:
+        assert float((want[p] - without[p]).abs().max()) > 0.2 * float(want.abs().max())
+    reqs = {"r0": tokens}
+    for what, trace in [("whole", H.trace_whole(reqs)), ("decoded", H.trace_last_decoded(reqs, 60)), ("portions", H.trace_portions(reqs))]:
+        eng = engine(path, dtype, page_size=16, max_tokens=704, max_requests=1)
+        rows = {k: v for k, v in H.replay(eng, trace).items() if k[1] >= 600}
+        H.assert_rows_match(rows, {"r0": want}, TOL[dtype], f"far key {dtype} {what}")
+
+
 def test_a_state_slot_that_is_used_again_starts_anew(models):
     """A request that takes the slot of a finished one gets what it gets in a new engine, bit for bit (float32): neither
     the matrices nor the convolutions' inputs of the request before reach it."""
