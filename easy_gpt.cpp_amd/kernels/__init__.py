@@ -82,6 +82,21 @@ Methods of a backend (T tokens, B requests, R rows, act = bfloat16 or float32):
         per request and head, token by token: S = diag(decay_t) S + k_t v_t^T, o_t = S^T (q_t * q_scale); S is read from and
         written to states[slots[b]] (fresh[b]: it starts at zero); q, k, v are columns of the product rows; the output comes as
         partial sums over ranges of the key channels (the backend's choice of S), which the consumer adds
+  (head_norm_store also takes row_width, cos_sin f32[T,rd/2,2] with rotary_dim and pairing 'half' | 'interleaved', norm_plain,
+   norm_after_rotation, values_are_keys; latent_prep takes queries (the query heads as a product of their own) and lead_width;
+   head_norm_gate takes gate_act 'silu' | 'sigmoid' | 'factor', x_width and x_act; normed_pair_mean without weights is
+   factor * a + factor_b * b; channel_decay takes rates f32[C] and negate: sigmoid(-z)^rates = exp(-rates * softplus(z));
+   decayed_state_scan takes k_silu, v_silu and head_decay f32[heads] in place of decay)
+  short_conv(proj, act_dtype, col0, conv_w act[C,taps], taps, unit_heads, unit_dim, scaled_heads, scale, unit_eps, sig_offset,
+             n_sig, states f32[slots,N], state_offset, slots i32[B], fresh bool[B]|None, q_start, q_len, max_q_len) -> f32[T,C+n_sig]
+        columns col0.. of the product rows through C causal convolutions over time (the last tap is the current token's; the
+        taps - 1 inputs before a step's first token come from states[slot, state_offset:] as [taps-1, C], zeros where fresh,
+        and that record is brought up to date), SiLU, the first unit_heads heads of unit_dim made unit vectors
+        (x / sqrt(sum x^2 + unit_eps), the first scaled_heads times scale); behind them sigmoid of n_sig further columns
+  delta_rule_scan(ops f32[T,W], q_offset, k_offset, v_offset, beta_offset, decay f32[T,heads*dk], states f32[slots,N],
+                  state_offset, slots, fresh, q_start, q_len, heads, kv_heads, dk, dv) -> f32[1,T,heads*dv]
+        per request and value head, token by token: S = diag(decay_t) S; u = beta_t (v_t - S^T k_t); S += k_t u^T; o_t = S^T q_t;
+        head h reads the queries and keys of head h // (heads // kv_heads); S [heads,dk,dv] lies at states[slot, state_offset:]
   expert_mixture(x act[T,H], router act[E,H], router_bias act[E]|None, w_gate_up act[E,2F,H], w_down act[E,H,F], top) -> f32[T,H]
         float32 logits x router^T + bias, the `top` largest (lowest index among equals), softmax over those; the weighted
         sum of down_e(silu(gate_e x) * (up_e x)) over the chosen experts e, added in the order of the choices
